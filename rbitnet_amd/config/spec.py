@@ -1,0 +1,67 @@
+"""Architecture-blind description of a model: which parts, in which order.
+
+A configuration class (one per architecture, see `llama.py`) turns its own
+config.json keys into a `ModelSpec`.  Everything below the configuration layer
+(the loader, the parts, the cache, the step function) reads only the spec, so no
+part knows which model it is in.
+
+A `PartSpec` is a kind name plus parameters; the kind is looked up in the part
+registries of `rbitnet_amd.parts`.  A `LayerSpec` holds the parts of one block
+and the prefix under which its tensors are stored.  `ModelSpec.schedule` is the
+order in which layers run: a list of indices into `layers`, which may name a
+layer twice.  A mixer whose parameters hold `cache_from = j` keeps no cache of
+its own and reads the one layer `j` wrote.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+
+@dataclass
+class PartSpec:
+    kind: str
+    params: Dict[str, Any] = field(default_factory=dict)
+
+    def __getitem__(self, key: str) -> Any:
+        return self.params[key]
+
+    def get(self, key: str, default: Any = None) -> Any:
+        return self.params.get(key, default)
+
+
+@dataclass
+class LayerSpec:
+    """One block.  `block` names the arrangement of the parts ("prenorm":
+    x += mixer(norm1(x)); x += ffn(norm2(x)))."""
+    prefix: str
+    block: str
+    mixer: PartSpec
+    feed_forward: PartSpec
+    norm1: PartSpec
+    norm2: PartSpec
+    # tensor-name segment of each part below `prefix`, e.g. {"mixer": "self_attn"}
+    segments: Optional[Dict[str, str]] = None
+
+
+@dataclass
+class ModelSpec:
+    architecture: str
+    hidden_size: int
+    vocab_size: int
+    max_positions: int
+    embedding_name: str
+    layers: List[LayerSpec]
+    final_norm: PartSpec
+    final_norm_name: str
+    head_name: Optional[str]          # None: the head is the embedding table (tied)
+    schedule: List[int] = field(default_factory=list)
+    stop_token_ids: List[int] = field(default_factory=list)
+    bos_token_id: Optional[int] = None
+
+    def __post_init__(self) -> None:
+        if not self.schedule:
+            self.schedule = list(range(len(self.layers)))
+        for i in self.schedule:
+            if not 0 <= i < len(self.layers):
+                raise ValueError(f"schedule names layer {i}, but the model has {len(self.layers)} layers")

@@ -1,0 +1,84 @@
+// C entry points of librbitnet_hip.so.  All pointers are device pointers unless a
+// name starts with h_.  Every function returns 0 on success; otherwise
+// rb_last_error() holds the reason.  `stream` is a hipStream_t.
+//
+// dtype codes: 0 = float32, 1 = bfloat16 (storage; arithmetic is float32 inside).
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* rb_last_error(void);
+int rb_version(void);
+int rb_page_size(void);
+
+// x[t, :] = table[ids[t], :] widened to float32.  ids are checked by the caller.
+int rb_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* x, int n_tokens, int width,
+                    void* stream);
+
+// Residual add and RMS norm in one pass.
+//   src = rows ? rows[r] : r
+//   v = x[src] + (delta ? delta[src] : 0);  if (delta && !rows) x[src] = v
+//   out[r] = v * gain * rsqrt(mean(v^2) + eps)
+int rb_add_rmsnorm(float* x, const float* delta, const float* gain, float eps, const int32_t* rows, int n_rows,
+                   int width, void* out, int out_dtype, void* stream);
+
+// Rotate q and k by the angle table, write q to q_out and k, v into the cache pages.
+//   qkv      float32 [T, (Hq + 2 Hk) D]: q heads, then k heads, then v heads
+//   cos, sin float32 [max_pos, D/2], or null for no rotation
+//   style    0: pairs (2i, 2i+1); 1: pairs (i, i + D/2)
+//   k_pages, v_pages [n_pages, Hk, 64, D] of cache_dtype; null when the layer keeps no cache
+//   tok_pos, tok_seq int32 [T]; block_table int32 [B, bt_stride]
+int rb_rope_kv_write(const float* qkv, const float* cos, const float* sin, int style, void* q_out, void* k_pages,
+                     void* v_pages, int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq,
+                     const int32_t* block_table, int bt_stride, int n_tokens, int n_heads, int n_kv_heads,
+                     int head_dim, void* stream);
+
+// t[r, j] = silu(gu[r, j]) * gu[r, F + j]
+int rb_swiglu(const float* gu, void* out, int out_dtype, int n_rows, int ff, void* stream);
+
+// C[M, N] = A[M, K] * W[N, K]^T with float32 accumulation; any sizes.
+int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dtype_out, int m, int n, int k,
+                    void* stream);
+
+// C[M, N] = A[M, K] * W[N, K]^T, bfloat16 inputs on the matrix cores.
+//   epilogue 0: store C (float32 or bfloat16)
+//   epilogue 1: W holds gate and up rows interleaved in blocks of 16
+//               (16 gate rows, then the 16 up rows of the same columns); the result is
+//               silu(gate) * up, [M, N/2]
+// K must be a multiple of 8 (rows 16-byte aligned).
+int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
+                 void* stream);
+
+// Causal attention of every token over its sequence's cache (keys 0..pos, or the last
+// `window` of them), any head_dim that is even and at most 256.
+//   q [T, Hq, D], out [T, Hq * D], both of dtype; pages as in rb_rope_kv_write.
+int rb_attention_generic(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype,
+                         const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table,
+                         int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int head_dim, float scale,
+                         int window, void* stream);
+
+// The same for bfloat16 and head_dim 64 or 128 on the matrix cores.
+//   prefill: sequences b = 0..B-1 hold tokens cu_seqlens[b]..cu_seqlens[b+1] at positions past_len[b]...
+int rb_attention_prefill_bf16(const void* q, const void* k_pages, const void* v_pages, void* out,
+                              const int32_t* cu_seqlens, const int32_t* past_len, const int32_t* block_table,
+                              int bt_stride, int n_seqs, int max_q_len, int n_heads, int n_kv_heads, int head_dim,
+                              float scale, int window, void* stream);
+//   decode: one token per sequence at position tok_pos[b]; the keys are split into
+//   n_splits ranges whose partial results are combined in a second kernel.
+//   workspace: float32 [B, Hq, n_splits, D + 2]
+int rb_attention_decode_bf16(const void* q, const void* k_pages, const void* v_pages, void* out,
+                             const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int n_seqs,
+                             int n_heads, int n_kv_heads, int head_dim, float scale, int window, int n_splits,
+                             float* workspace, void* stream);
+
+// tokens[r] = argmax of logits[r, :] (NaN counts as -inf, lowest index among equals), or, where
+// temperature[r] > 0, the first index whose running sum of exp(z/T - max) reaches u[r] times the total.
+int rb_sample(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,
+              int32_t* tokens, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,474 @@
+// Attention over the paged cache for bfloat16 and head sizes 64 and 128.
+//
+//  * prefill: causal flash attention on the matrix cores.  A workgroup of 4 waves takes
+//    one kv head and 32-query blocks of the query heads that share it; the 64-key page
+//    tiles of K and V are staged through LDS once for all of them.  Scores are computed
+//    transposed (keys x queries) so that the probabilities come out of the first MFMA in
+//    the lane layout the second one wants; V is transposed on its way into LDS.
+//  * decode: one query per sequence.  The pages of a sequence are dealt out to n_splits
+//    workgroups per kv head, each keeps a running softmax for the query heads of its kv
+//    head, and a second kernel combines the splits.
+//
+// Scores, maxima, exponentials, sums and the output accumulators are float32; the
+// probabilities are rounded to bfloat16 for the second MFMA in prefill only.
+//
+// Reference: s[p] = (q . K[p]) / sqrt(D) for p <= pos, softmax with the maximum
+// subtracted, out = sum_p s[p] V[p]; q head qh reads kv head qh / (Hq / Hk)
+// (llama/model.rs:260-289, softmax :102-114).
+#include <math.h>
+
+#include "api.h"
+#include "mfma.h"
+
+#define LOG2E 1.4426950408889634f
+
+// =============================================================================== prefill
+template <int D>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    bf16_t* __restrict__ out, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ past_len,
+    const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, float scale_log2, int window,
+    int gw) {
+  constexpr int KLD = D + 8;          // K tile row: D + 8 elements, rows 16 bytes apart in bank space
+  constexpr int VLD = RB_PAGE + 8;    // V^T tile row: 64 keys + 8
+  constexpr int DC = D / 8;           // 16-byte chunks per row
+  constexpr int KCH = RB_PAGE * DC / 256;
+  __shared__ __attribute__((aligned(16))) bf16_t ks[RB_PAGE * KLD];
+  __shared__ __attribute__((aligned(16))) bf16_t vt[D * VLD];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int b = blockIdx.z;
+  const int group = n_heads / n_kv;
+  const int groups_per_kv = group / gw;
+  const int kvh = blockIdx.y / groups_per_kv;
+  const int head = kvh * group + (blockIdx.y % groups_per_kv) * gw + (wave % gw);
+  const int q_per_wg = 32 * (4 / gw);
+  const int seq_start = cu_seqlens[b];
+  const int q_len = cu_seqlens[b + 1] - seq_start;
+  const int past = past_len[b];
+  const int wg_q0 = blockIdx.x * q_per_wg;
+  if (wg_q0 >= q_len) return;
+  const int q0 = wg_q0 + (wave / gw) * 32;
+  const bool wave_on = q0 < q_len;
+  const int kv_last = past + q_len - 1;                       // last key this sequence holds
+
+  // ---- this lane's query
+  int ql = q0 + l32;
+  const bool q_ok = ql < q_len;
+  if (ql >= q_len) ql = q_len - 1;
+  const int qpos = past + ql;
+  const int q_lo = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
+  Frag8 qf[D / 16];
+  {
+    const bf16_t* qrow = q + ((size_t)(seq_start + ql) * n_heads + head) * D;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) qf[s].u = load16(qrow + s * 16 + g * 8);
+  }
+
+  // ---- key tiles of the workgroup and of this wave
+  const int wg_q_end = (wg_q0 + q_per_wg < q_len ? wg_q0 + q_per_wg : q_len) - 1;
+  const int wg_min_pos = past + wg_q0;
+  const int wg_lo = (window > 0 && wg_min_pos - window + 1 > 0) ? wg_min_pos - window + 1 : 0;
+  const int first_tile = wg_lo / RB_PAGE;
+  const int last_tile = (past + wg_q_end) / RB_PAGE;
+  int wave_first = first_tile, wave_last = -1;
+  if (wave_on) {
+    const int w_end = (q0 + 32 < q_len ? q0 + 32 : q_len) - 1;
+    wave_last = (past + w_end) / RB_PAGE;
+    const int w_min = past + q0;
+    wave_first = ((window > 0 && w_min - window + 1 > 0) ? w_min - window + 1 : 0) / RB_PAGE;
+  }
+
+  float m_run = -INFINITY, l_run = 0.f;
+  f32x16_t oacc[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[i][e] = 0.f;
+
+  // ---- staging roles
+  // V: a thread takes 4 consecutive keys x 8 consecutive d (one 16-byte chunk of 4 rows)
+  const int v_dchunk = (tid & 3) + 4 * (tid >> 6);
+  const int v_quad = (tid >> 2) & 15;
+  const bool v_on = v_dchunk < DC;
+  // place of the quad in the permuted key order of a V^T row (see the second MFMA below)
+  const int qq = v_quad & 7;
+  const int v_col = (v_quad >> 3) * 32 + (2 * (qq >> 2) + (qq & 1)) * 8 + ((qq >> 1) & 1) * 4;
+
+  uint4 kreg[KCH], vreg[4];
+  auto load_tile = [&](int kt) {
+    const int page = block_table[(size_t)b * bt_stride + kt];
+    const size_t base = ((size_t)page * n_kv + kvh) * RB_PAGE * D;
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + 256 * i;
+      kreg[i] = load16(k_pages + base + (size_t)(c / DC) * D + (c % DC) * 8);
+    }
+    if (v_on) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int key = kt * RB_PAGE + 4 * v_quad + e;
+        // keys outside what the sequence holds may be anything, even NaN: make them zero
+        vreg[e] = (key <= kv_last && key >= wg_lo) ? load16(v_pages + base + (size_t)(4 * v_quad + e) * D + v_dchunk * 8)
+                                                   : zero16();
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + 256 * i;
+      *reinterpret_cast<uint4*>(ks + (c / DC) * KLD + (c % DC) * 8) = kreg[i];
+    }
+    if (v_on) {
+      const uint32_t w0[4] = {vreg[0].x, vreg[1].x, vreg[2].x, vreg[3].x};
+      const uint32_t w1[4] = {vreg[0].y, vreg[1].y, vreg[2].y, vreg[3].y};
+      const uint32_t w2[4] = {vreg[0].z, vreg[1].z, vreg[2].z, vreg[3].z};
+      const uint32_t w3[4] = {vreg[0].w, vreg[1].w, vreg[2].w, vreg[3].w};
+      auto put = [&](int i, const uint32_t* w, bool hi) {
+        uint2 o;
+        if (!hi) {
+          o.x = (w[0] & 0xffffu) | (w[1] << 16);
+          o.y = (w[2] & 0xffffu) | (w[3] << 16);
+        } else {
+          o.x = (w[0] >> 16) | (w[1] & 0xffff0000u);
+          o.y = (w[2] >> 16) | (w[3] & 0xffff0000u);
+        }
+        *reinterpret_cast<uint2*>(vt + (v_dchunk * 8 + i) * VLD + v_col) = o;
+      };
+      put(0, w0, false);
+      put(1, w0, true);
+      put(2, w1, false);
+      put(3, w1, true);
+      put(4, w2, false);
+      put(5, w2, true);
+      put(6, w3, false);
+      put(7, w3, true);
+    }
+  };
+
+  load_tile(first_tile);
+  for (int kt = first_tile; kt <= last_tile; ++kt) {
+    __syncthreads();                 // everyone is done reading the previous tile
+    store_tile();
+    __syncthreads();
+    if (kt + 1 <= last_tile) load_tile(kt + 1);
+    if (!(wave_on && kt >= wave_first && kt <= wave_last)) continue;
+
+    // ---- S^T = K Q^T: rows keys, columns queries
+    f32x16_t sacc[2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sacc[rt][e] = 0.f;
+#pragma unroll
+      for (int s = 0; s < D / 16; ++s) {
+        Frag8 a;
+        a.u = *reinterpret_cast<const uint4*>(ks + (rt * 32 + l32) * KLD + s * 16 + g * 8);
+        sacc[rt] = mfma32(a, qf[s], sacc[rt]);
+      }
+    }
+    // ---- mask, running maximum
+    float mx = -INFINITY;
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int key = kt * RB_PAGE + rt * 32 + 8 * (e / 4) + 4 * g + (e % 4);
+        float s = sacc[rt][e] * scale_log2;
+        if (key > qpos || key < q_lo) s = -INFINITY;
+        sacc[rt][e] = s;
+        mx = fmaxf(mx, s);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = exp2f(m_run - m_safe);          // m_run = -inf gives 0
+    float lsum = 0.f;
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float p = exp2f(sacc[rt][e] - m_safe);
+        sacc[rt][e] = p;
+        lsum += p;
+      }
+    lsum += __shfl_xor(lsum, 32, 64);
+    l_run = l_run * corr + lsum;
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) oacc[i][e] *= corr;
+
+    // ---- O^T += V^T P^T.  Step (rt, mm) takes the 16 keys whose probabilities sit in
+    // registers 8 mm .. 8 mm + 7 of row tile rt: for lane group g these are keys
+    // 32 rt + 16 mm + 8 h + 4 g + e (h = 0, 1; e = 0..3), and V^T was stored in that order.
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int mm = 0; mm < 2; ++mm) {
+        Frag8 pb;
+        pb.u.x = pack_bf16x2(sacc[rt][8 * mm + 0], sacc[rt][8 * mm + 1]);
+        pb.u.y = pack_bf16x2(sacc[rt][8 * mm + 2], sacc[rt][8 * mm + 3]);
+        pb.u.z = pack_bf16x2(sacc[rt][8 * mm + 4], sacc[rt][8 * mm + 5]);
+        pb.u.w = pack_bf16x2(sacc[rt][8 * mm + 6], sacc[rt][8 * mm + 7]);
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i) {
+          Frag8 a;
+          a.u = *reinterpret_cast<const uint4*>(vt + (i * 32 + l32) * VLD + rt * 32 + (2 * mm + g) * 8);
+          oacc[i] = mfma32(a, pb, oacc[i]);
+        }
+      }
+  }
+
+  if (!wave_on || !q_ok) return;
+  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  bf16_t* orow = out + ((size_t)(seq_start + ql) * n_heads + head) * D;
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+    for (int e4 = 0; e4 < 4; ++e4) {
+      uint2 o;
+      o.x = pack_bf16x2(oacc[i][4 * e4 + 0] * inv, oacc[i][4 * e4 + 1] * inv);
+      o.y = pack_bf16x2(oacc[i][4 * e4 + 2] * inv, oacc[i][4 * e4 + 3] * inv);
+      *reinterpret_cast<uint2*>(orow + i * 32 + 8 * e4 + 4 * g) = o;
+    }
+}
+
+extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                         const int32_t* cu_seqlens, const int32_t* past_len,
+                                         const int32_t* block_table, int bt_stride, int n_seqs, int max_q_len,
+                                         int n_heads, int n_kv_heads, int head_dim, float scale, int window,
+                                         void* stream) {
+  RB_REQUIRE(n_seqs > 0 && max_q_len > 0, "rb_attention_prefill_bf16: empty batch");
+  RB_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+             "rb_attention_prefill_bf16: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
+  RB_REQUIRE(head_dim == 64 || head_dim == 128,
+             "rb_attention_prefill_bf16: head_dim %d not supported (64 or 128; use rb_attention_generic)", head_dim);
+  RB_REQUIRE(window >= 0, "rb_attention_prefill_bf16: negative window");
+  const int group = n_heads / n_kv_heads;
+  const int gw = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+  const int q_per_wg = 32 * (4 / gw);
+  dim3 grid((max_q_len + q_per_wg - 1) / q_per_wg, n_kv_heads * (group / gw), n_seqs);
+  RB_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "rb_attention_prefill_bf16: batch or head count too large");
+  hipStream_t s = (hipStream_t)stream;
+  const float sl2 = scale * LOG2E;
+  if (head_dim == 128)
+    attn_prefill_kernel<128><<<grid, 256, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
+                                                 (bf16_t*)out, cu_seqlens, past_len, block_table, bt_stride,
+                                                 n_heads, n_kv_heads, sl2, window, gw);
+  else
+    attn_prefill_kernel<64><<<grid, 256, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
+                                                (bf16_t*)out, cu_seqlens, past_len, block_table, bt_stride,
+                                                n_heads, n_kv_heads, sl2, window, gw);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// =============================================================================== decode
+template <int D, int G>
+__global__ __launch_bounds__(256) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
+    int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws) {
+  constexpr int DL = D / 64;          // output elements per lane
+  constexpr int QC = D / 32;          // 16-byte chunks of a quarter row of K
+  __shared__ float q_s[G][D];
+  __shared__ float p_s[4][G][16];
+  __shared__ float red_m[4][G], red_l[4][G];
+  __shared__ float red_acc[4][G][D];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int pos = tok_pos[b];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first_page = lo / RB_PAGE, last_page = pos / RB_PAGE;
+
+  for (int idx = tid; idx < G * D; idx += 256) {
+    const int gg = idx / D, d = idx % D;
+    q_s[gg][d] = bf16_to_f32(q[((size_t)b * n_heads + kvh * G + gg) * D + d]) * scale_log2;
+  }
+  __syncthreads();
+
+  float m_run[G], l_run[G], acc[G][DL];
+#pragma unroll
+  for (int gg = 0; gg < G; ++gg) {
+    m_run[gg] = -INFINITY;
+    l_run[gg] = 0.f;
+#pragma unroll
+    for (int e = 0; e < DL; ++e) acc[gg][e] = 0.f;
+  }
+  const int j = lane >> 2, part = lane & 3;
+  for (int pg = first_page + split; pg <= last_page; pg += n_splits) {
+    const int page = block_table[(size_t)b * bt_stride + pg];
+    const size_t base = ((size_t)page * n_kv + kvh) * RB_PAGE * D;
+    const int key0 = pg * RB_PAGE + wave * 16;
+    const int key = key0 + j;
+    const bool valid = key >= lo && key <= pos;
+    // ---- scores: lane (j, part) takes a quarter of key j's row
+    float s[G];
+#pragma unroll
+    for (int gg = 0; gg < G; ++gg) s[gg] = 0.f;
+    const bf16_t* krow = k_pages + base + (size_t)(wave * 16 + j) * D + part * (D / 4);
+#pragma unroll
+    for (int cidx = 0; cidx < QC; ++cidx) {
+      const uint4 u = load16(krow + cidx * 8);
+      const uint32_t wds[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float k0 = bf16_bits_to_f32(wds[e] & 0xffffu);
+        const float k1 = bf16_bits_to_f32(wds[e] >> 16);
+        const int d = part * (D / 4) + cidx * 8 + 2 * e;
+#pragma unroll
+        for (int gg = 0; gg < G; ++gg) s[gg] = fmaf(k1, q_s[gg][d + 1], fmaf(k0, q_s[gg][d], s[gg]));
+      }
+    }
+#pragma unroll
+    for (int gg = 0; gg < G; ++gg) {
+      float v = s[gg];
+      v += __shfl_xor(v, 1, 64);
+      v += __shfl_xor(v, 2, 64);
+      if (!valid) v = -INFINITY;
+      float mx = v;
+#pragma unroll
+      for (int o = 4; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      const float m_new = fmaxf(m_run[gg], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float corr = exp2f(m_run[gg] - m_safe);
+      const float p = exp2f(v - m_safe);
+      float ps = p;
+#pragma unroll
+      for (int o = 4; o < 64; o <<= 1) ps += __shfl_xor(ps, o, 64);
+      l_run[gg] = l_run[gg] * corr + ps;
+      m_run[gg] = m_new;
+#pragma unroll
+      for (int e = 0; e < DL; ++e) acc[gg][e] *= corr;
+      if (part == 0) p_s[wave][gg][j] = p;
+    }
+    __syncthreads();
+    // ---- weighted sum of the values: lane takes DL consecutive d
+    int jj_lo = lo - key0;
+    if (jj_lo < 0) jj_lo = 0;
+    int jj_hi = pos - key0;
+    if (jj_hi > 15) jj_hi = 15;
+    const bf16_t* vcol = v_pages + base + (size_t)(wave * 16) * D + lane * DL;
+    for (int jj = jj_lo; jj <= jj_hi; ++jj) {
+      float v[DL];
+      if (DL == 2) {
+        const uint32_t u = *reinterpret_cast<const uint32_t*>(vcol + (size_t)jj * D);
+        v[0] = bf16_bits_to_f32(u & 0xffffu);
+        v[DL - 1] = bf16_bits_to_f32(u >> 16);
+      } else {
+        v[0] = bf16_to_f32(vcol[(size_t)jj * D]);
+      }
+#pragma unroll
+      for (int gg = 0; gg < G; ++gg) {
+        const float p = p_s[wave][gg][jj];
+#pragma unroll
+        for (int e = 0; e < DL; ++e) acc[gg][e] = fmaf(p, v[e], acc[gg][e]);
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- combine the four waves, write this split's partial result
+#pragma unroll
+  for (int gg = 0; gg < G; ++gg) {
+    if (lane == 0) {
+      red_m[wave][gg] = m_run[gg];
+      red_l[wave][gg] = l_run[gg];
+    }
+#pragma unroll
+    for (int e = 0; e < DL; ++e) red_acc[wave][gg][lane * DL + e] = acc[gg][e];
+  }
+  __syncthreads();
+  for (int idx = tid; idx < G * D; idx += 256) {
+    const int gg = idx / D, d = idx % D;
+    float mx = red_m[0][gg];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) mx = fmaxf(mx, red_m[w][gg]);
+    const float m_safe = (mx == -INFINITY) ? 0.f : mx;
+    float a = 0.f, l = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = exp2f(red_m[w][gg] - m_safe);
+      a += red_acc[w][gg][d] * f;
+      l += red_l[w][gg] * f;
+    }
+    float* dst = ws + (((size_t)b * n_heads + kvh * G + gg) * n_splits + split) * (D + 2);
+    dst[d] = a;
+    if (d == 0) {
+      dst[D] = mx;
+      dst[D + 1] = l;
+    }
+  }
+}
+
+template <int D>
+__global__ void attn_decode_combine_kernel(const float* __restrict__ ws, bf16_t* __restrict__ out, int n_splits) {
+  const size_t row = blockIdx.x;            // sequence * heads + head
+  const int d = threadIdx.x;
+  const float* src = ws + row * n_splits * (D + 2);
+  float mx = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, src[(size_t)s * (D + 2) + D]);
+  const float m_safe = (mx == -INFINITY) ? 0.f : mx;
+  float a = 0.f, l = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float f = exp2f(src[(size_t)s * (D + 2) + D] - m_safe);
+    a += src[(size_t)s * (D + 2) + d] * f;
+    l += src[(size_t)s * (D + 2) + D + 1] * f;
+  }
+  out[row * D + d] = f32_to_bf16(l > 0.f ? a / l : 0.f);
+}
+
+template <int D, int G>
+static void launch_decode(const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* out, const int32_t* tok_pos,
+                          const int32_t* bt, int bt_stride, int n_seqs, int n_heads, int n_kv, float sl2, int window,
+                          int n_splits, float* ws, hipStream_t s) {
+  dim3 grid(n_splits, n_kv, n_seqs);
+  attn_decode_kernel<D, G><<<grid, 256, 0, s>>>(q, k, v, tok_pos, bt, bt_stride, n_heads, n_kv, sl2, window,
+                                                n_splits, ws);
+  attn_decode_combine_kernel<D><<<n_seqs * n_heads, D, 0, s>>>(ws, out, n_splits);
+}
+
+extern "C" int rb_attention_decode_bf16(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                        const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
+                                        int n_seqs, int n_heads, int n_kv_heads, int head_dim, float scale,
+                                        int window, int n_splits, float* workspace, void* stream) {
+  RB_REQUIRE(n_seqs > 0, "rb_attention_decode_bf16: empty batch");
+  RB_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+             "rb_attention_decode_bf16: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
+  RB_REQUIRE(head_dim == 64 || head_dim == 128,
+             "rb_attention_decode_bf16: head_dim %d not supported (64 or 128; use rb_attention_generic)", head_dim);
+  RB_REQUIRE(n_splits >= 1 && n_splits <= 65535, "rb_attention_decode_bf16: bad split count %d", n_splits);
+  RB_REQUIRE(n_kv_heads <= 65535 && n_seqs <= 65535, "rb_attention_decode_bf16: batch or head count too large");
+  RB_REQUIRE(window >= 0, "rb_attention_decode_bf16: negative window");
+  const int group = n_heads / n_kv_heads;
+  RB_REQUIRE(group == 1 || group == 2 || group == 4 || group == 8,
+             "rb_attention_decode_bf16: %d query heads per kv head not supported (1, 2, 4, 8; use "
+             "rb_attention_generic)", group);
+  hipStream_t s = (hipStream_t)stream;
+  const float sl2 = scale * LOG2E;
+  const bf16_t* qq = (const bf16_t*)q;
+  const bf16_t* kk = (const bf16_t*)k_pages;
+  const bf16_t* vv = (const bf16_t*)v_pages;
+  bf16_t* oo = (bf16_t*)out;
+#define RB_DEC(DV, GV)                                                                                         \
+  launch_decode<DV, GV>(qq, kk, vv, oo, tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, sl2, window, \
+                        n_splits, workspace, s)
+  if (head_dim == 128) {
+    if (group == 1) RB_DEC(128, 1);
+    else if (group == 2) RB_DEC(128, 2);
+    else if (group == 4) RB_DEC(128, 4);
+    else RB_DEC(128, 8);
+  } else {
+    if (group == 1) RB_DEC(64, 1);
+    else if (group == 2) RB_DEC(64, 2);
+    else if (group == 4) RB_DEC(64, 4);
+    else RB_DEC(64, 8);
+  }
+#undef RB_DEC
+  RB_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,94 @@
+// Shared device helpers for the gfx950 kernels: storage types, wave and block
+// reductions, error reporting of the C entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define RB_WAVE 64
+#define RB_PAGE 64            // tokens per cache page; attention tiles are one page of keys
+
+// ---------------------------------------------------------------- error reporting
+// Every entry point returns 0, or a non-zero code after rb_set_error(); the text is
+// read back with rb_last_error().  No entry point throws or aborts.
+void rb_set_error(const char* fmt, ...);
+#define RB_REQUIRE(cond, ...)                       \
+  do {                                              \
+    if (!(cond)) {                                  \
+      rb_set_error(__VA_ARGS__);                    \
+      return 1;                                     \
+    }                                               \
+  } while (0)
+#define RB_LAUNCH_CHECK()                                                   \
+  do {                                                                      \
+    hipError_t e_ = hipGetLastError();                                      \
+    if (e_ != hipSuccess) {                                                 \
+      rb_set_error("%s: launch failed: %s", __func__, hipGetErrorString(e_)); \
+      return 2;                                                             \
+    }                                                                       \
+  } while (0)
+
+enum RbDtype { RB_F32 = 0, RB_BF16 = 1 };
+
+// ---------------------------------------------------------------- bfloat16 storage
+struct bf16_t {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  bf16_t r;
+  r.bits = f32_to_bf16_bits(f);
+  return r;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+
+template <typename T>
+struct Num;
+template <>
+struct Num<float> {
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <>
+struct Num<bf16_t> {
+  static __device__ __forceinline__ float load(const bf16_t* p) { return bf16_to_f32(*p); }
+  static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+};
+
+// ---------------------------------------------------------------- reductions
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = RB_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, RB_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = RB_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, RB_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; `scratch` holds at least 16 floats.
+// Every thread gets the total.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (RB_WAVE - 1);
+  const int wave = threadIdx.x / RB_WAVE;
+  const int n_waves = (blockDim.x + RB_WAVE - 1) / RB_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < n_waves; ++i) t += scratch[i];
+  return t;
+}

@@ -1,0 +1,209 @@
+// Embedding gather, fused residual-add + RMS norm, rotary encoding with cache write,
+// SiLU gate.  All arithmetic in float32; storage float32 or bfloat16.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "api.h"
+#include "common.h"
+
+// ---------------------------------------------------------------- errors
+static thread_local char g_error[512];
+void rb_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+extern "C" const char* rb_last_error(void) { return g_error; }
+extern "C" int rb_version(void) { return 1; }
+extern "C" int rb_page_size(void) { return RB_PAGE; }
+
+// ---------------------------------------------------------------- embedding
+// Reference: x[j] = token_embd[j + tok * n_embd] (llama/model.rs:229-232).
+template <typename T>
+__global__ void embed_gather_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
+                                    float* __restrict__ x, int width) {
+  const int t = blockIdx.x;
+  const T* row = table + (size_t)ids[t] * width;
+  float* dst = x + (size_t)t * width;
+  for (int j = threadIdx.x; j < width; j += blockDim.x) dst[j] = Num<T>::load(row + j);
+}
+
+extern "C" int rb_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* x, int n_tokens,
+                               int width, void* stream) {
+  RB_REQUIRE(n_tokens >= 0 && width > 0, "rb_embed_gather: bad sizes %d x %d", n_tokens, width);
+  if (n_tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (table_dtype == RB_F32)
+    embed_gather_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)table, ids, x, width);
+  else if (table_dtype == RB_BF16)
+    embed_gather_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)table, ids, x, width);
+  else
+    RB_REQUIRE(false, "rb_embed_gather: unknown dtype %d", table_dtype);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- add + rmsnorm
+// Reference: s = sum(x^2)/n; scale = 1/sqrt(s + eps); y = x * w * scale
+// (llama/model.rs:93-100); residual adds are plain sums (:292-294, :304-306).
+template <typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ delta,
+                                   const float* __restrict__ gain, float eps, const int32_t* __restrict__ rows,
+                                   int width, TO* __restrict__ out) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* xr = x + src * width;
+  const float* dr = delta ? delta + src * width : nullptr;
+  const bool write_back = (delta != nullptr) && (rows == nullptr);
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < width; j += blockDim.x) {
+    float v = xr[j];
+    if (dr) v += dr[j];
+    if (write_back) xr[j] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)width + eps);
+  TO* orow = out + (size_t)r * width;
+  for (int j = threadIdx.x; j < width; j += blockDim.x) {
+    float v = xr[j];
+    if (dr && !write_back) v += dr[j];
+    Num<TO>::store(orow + j, v * gain[j] * scale);
+  }
+}
+
+extern "C" int rb_add_rmsnorm(float* x, const float* delta, const float* gain, float eps, const int32_t* rows,
+                              int n_rows, int width, void* out, int out_dtype, void* stream) {
+  RB_REQUIRE(n_rows >= 0 && width > 0, "rb_add_rmsnorm: bad sizes %d x %d", n_rows, width);
+  if (n_rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = width >= 2048 ? 512 : 256;
+  if (out_dtype == RB_F32)
+    add_rmsnorm_kernel<float><<<n_rows, threads, 0, s>>>(x, delta, gain, eps, rows, width, (float*)out);
+  else if (out_dtype == RB_BF16)
+    add_rmsnorm_kernel<bf16_t><<<n_rows, threads, 0, s>>>(x, delta, gain, eps, rows, width, (bf16_t*)out);
+  else
+    RB_REQUIRE(false, "rb_add_rmsnorm: unknown dtype %d", out_dtype);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- rope + cache write
+// Reference: for i < D/2 the pair is rotated by pos * inv_i,
+//   x0' = x0 cos - x1 sin, x1' = x0 sin + x1 cos (llama/model.rs:122-136), for every q
+// head and k head (:242-252); k is cached rotated, v as it is (:254-257).
+template <typename TC>
+__global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const float* __restrict__ cos_t,
+                                     const float* __restrict__ sin_t, int style, TC* __restrict__ q_out,
+                                     TC* __restrict__ k_pages, TC* __restrict__ v_pages,
+                                     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
+                                     const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
+                                     int n_kv, int head_dim) {
+  const int t = blockIdx.x;
+  const int pos = tok_pos[t];
+  const int half = head_dim / 2;
+  const int row_width = (n_heads + 2 * n_kv) * head_dim;
+  const float* src = qkv + (size_t)t * row_width;
+  const float* cr = cos_t ? cos_t + (size_t)pos * half : nullptr;
+  const float* sr = sin_t ? sin_t + (size_t)pos * half : nullptr;
+  size_t page_base = 0;
+  if (k_pages) {
+    const int page = block_table[(size_t)tok_seq[t] * bt_stride + pos / RB_PAGE];
+    page_base = ((size_t)page * n_kv) * RB_PAGE * head_dim + (size_t)(pos % RB_PAGE) * head_dim;
+  }
+  // rotated pairs: q heads and k heads
+  const int n_rot = (n_heads + n_kv) * half;
+  for (int idx = threadIdx.x; idx < n_rot; idx += blockDim.x) {
+    const int h = idx / half;
+    const int i = idx - h * half;
+    const int i0 = style == 0 ? 2 * i : i;
+    const int i1 = style == 0 ? 2 * i + 1 : i + half;
+    const float x0 = src[h * head_dim + i0];
+    const float x1 = src[h * head_dim + i1];
+    float y0 = x0, y1 = x1;
+    if (cr) {
+      const float c = cr[i], s = sr[i];
+      y0 = x0 * c - x1 * s;
+      y1 = x0 * s + x1 * c;
+    }
+    if (h < n_heads) {
+      TC* dst = q_out + ((size_t)t * n_heads + h) * head_dim;
+      Num<TC>::store(dst + i0, y0);
+      Num<TC>::store(dst + i1, y1);
+    } else if (k_pages) {
+      TC* dst = k_pages + page_base + (size_t)(h - n_heads) * RB_PAGE * head_dim;
+      Num<TC>::store(dst + i0, y0);
+      Num<TC>::store(dst + i1, y1);
+    }
+  }
+  if (v_pages) {
+    const float* vsrc = src + (size_t)(n_heads + n_kv) * head_dim;
+    for (int idx = threadIdx.x; idx < n_kv * head_dim; idx += blockDim.x) {
+      const int h = idx / head_dim;
+      const int d = idx - h * head_dim;
+      Num<TC>::store(v_pages + page_base + (size_t)h * RB_PAGE * head_dim + d, vsrc[idx]);
+    }
+  }
+}
+
+extern "C" int rb_rope_kv_write(const float* qkv, const float* cos, const float* sin, int style, void* q_out,
+                                void* k_pages, void* v_pages, int cache_dtype, const int32_t* tok_pos,
+                                const int32_t* tok_seq, const int32_t* block_table, int bt_stride, int n_tokens,
+                                int n_heads, int n_kv_heads, int head_dim, void* stream) {
+  RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0 && head_dim % 2 == 0,
+             "rb_rope_kv_write: bad sizes T=%d Hq=%d Hk=%d D=%d", n_tokens, n_heads, n_kv_heads, head_dim);
+  RB_REQUIRE((cos == nullptr) == (sin == nullptr), "rb_rope_kv_write: cos and sin tables go together");
+  RB_REQUIRE(style == 0 || style == 1, "rb_rope_kv_write: unknown pairing style %d", style);
+  RB_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rb_rope_kv_write: k and v pages go together");
+  if (n_tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (cache_dtype == RB_F32)
+    rope_kv_write_kernel<float><<<n_tokens, 256, 0, s>>>(qkv, cos, sin, style, (float*)q_out, (float*)k_pages,
+                                                         (float*)v_pages, tok_pos, tok_seq, block_table,
+                                                         bt_stride, n_heads, n_kv_heads, head_dim);
+  else if (cache_dtype == RB_BF16)
+    rope_kv_write_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(qkv, cos, sin, style, (bf16_t*)q_out,
+                                                          (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, tok_seq,
+                                                          block_table, bt_stride, n_heads, n_kv_heads, head_dim);
+  else
+    RB_REQUIRE(false, "rb_rope_kv_write: unknown dtype %d", cache_dtype);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- SiLU gate
+// Reference: silu(v) = v / (1 + exp(-v)); t = silu(gate) * up (llama/model.rs:116-120, 297-302).
+template <typename TO>
+__global__ void swiglu_kernel(const float* __restrict__ gu, TO* __restrict__ out, int ff) {
+  const size_t r = blockIdx.y;
+  const float* g = gu + r * 2 * (size_t)ff;
+  const float* u = g + ff;
+  TO* o = out + r * (size_t)ff;
+  for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < ff; j += gridDim.x * blockDim.x) {
+    const float gv = g[j];
+    Num<TO>::store(o + j, gv / (1.0f + expf(-gv)) * u[j]);
+  }
+}
+
+extern "C" int rb_swiglu(const float* gu, void* out, int out_dtype, int n_rows, int ff, void* stream) {
+  RB_REQUIRE(n_rows >= 0 && ff > 0, "rb_swiglu: bad sizes %d x %d", n_rows, ff);
+  RB_REQUIRE(n_rows <= 65535 * 64, "rb_swiglu: too many rows %d", n_rows);
+  if (n_rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  // rows go to grid.y in chunks so that any row count fits the launch limits
+  for (int r0 = 0; r0 < n_rows; r0 += 65535) {
+    const int nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
+    dim3 grid((ff + 255) / 256 < 64 ? (ff + 255) / 256 : 64, nr);
+    const float* src = gu + (size_t)r0 * 2 * ff;
+    if (out_dtype == RB_F32)
+      swiglu_kernel<float><<<grid, 256, 0, s>>>(src, (float*)out + (size_t)r0 * ff, ff);
+    else if (out_dtype == RB_BF16)
+      swiglu_kernel<bf16_t><<<grid, 256, 0, s>>>(src, (bf16_t*)out + (size_t)r0 * ff, ff);
+    else
+      RB_REQUIRE(false, "rb_swiglu: unknown dtype %d", out_dtype);
+  }
+  RB_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,85 @@
+// C[M, N] = A[M, K] * W[N, K]^T for any sizes, float32 or bfloat16 storage, float32
+// multiply-add on the vector units (never a reduced-precision matrix mode).  This is the
+// whole float32 path's matrix product and the bfloat16 path's product for shapes the
+// matrix-core kernels refuse.
+//
+// Reference: y[o] = sum_i W[i + o * n_in] * x[i] (llama/model.rs:67-91).
+#include "api.h"
+#include "common.h"
+
+#define GT 64      // tile of C: GT x GT
+#define GK 16      // depth of one stage
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const TI* __restrict__ a, const TI* __restrict__ w,
+                                                           TO* __restrict__ c, int m, int n, int k) {
+  __shared__ float as[GK][GT + 4];
+  __shared__ float ws[GK][GT + 4];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.y * GT;
+  const int n0 = blockIdx.x * GT;
+  const int tx = tid % 16;      // 4 columns of C each
+  const int ty = tid / 16;      // 4 rows of C each
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  // each thread loads 4 elements of the A tile and 4 of the W tile per stage
+  const int lr = tid / 4;            // row of the tile, 0..63
+  const int lk = (tid % 4) * 4;      // depth offset 0, 4, 8, 12
+  for (int k0 = 0; k0 < k; k0 += GK) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int kk = k0 + lk + q;
+      const int am = m0 + lr;
+      const int wn = n0 + lr;
+      as[lk + q][lr] = (am < m && kk < k) ? Num<TI>::load(a + (size_t)am * k + kk) : 0.f;
+      ws[lk + q][lr] = (wn < n && kk < k) ? Num<TI>::load(w + (size_t)wn * k + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < GK; ++kk) {
+      float av[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = as[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wv[j] = ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int mm = m0 + ty * 4 + i;
+    if (mm >= m) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int nn = n0 + tx * 4 + j;
+      if (nn < n) Num<TO>::store(c + (size_t)mm * n + nn, acc[i][j]);
+    }
+  }
+}
+
+extern "C" int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dtype_out, int m, int n,
+                               int k, void* stream) {
+  RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_generic: bad sizes M=%d N=%d K=%d", m, n, k);
+  if (m == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((n + GT - 1) / GT, (m + GT - 1) / GT);
+  RB_REQUIRE(grid.y <= 65535, "rb_gemm_generic: M=%d too large for one launch", m);
+  if (dtype_in == RB_F32 && dtype_out == RB_F32)
+    gemm_generic_kernel<float, float><<<grid, 256, 0, s>>>((const float*)a, (const float*)w, (float*)c, m, n, k);
+  else if (dtype_in == RB_BF16 && dtype_out == RB_F32)
+    gemm_generic_kernel<bf16_t, float><<<grid, 256, 0, s>>>((const bf16_t*)a, (const bf16_t*)w, (float*)c, m, n, k);
+  else if (dtype_in == RB_BF16 && dtype_out == RB_BF16)
+    gemm_generic_kernel<bf16_t, bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)c, m, n, k);
+  else
+    RB_REQUIRE(false, "rb_gemm_generic: unsupported dtypes in=%d out=%d", dtype_in, dtype_out);
+  RB_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,354 @@
+// C[M, N] = A[M, K] * W[N, K]^T for bfloat16 operands on the gfx950 matrix cores, float32
+// accumulation.  W rows are the row operand of the MFMA and the tokens its columns, so a
+// lane ends up with 4 (or 8) consecutive outputs of one token.
+//
+// Two kernels:
+//  * skinny (M <= 64, decode): bound by reading W once.  A wave owns 16*R rows of W and a
+//    slice of K, streams them with 16-byte loads straight into MFMA operands, and the
+//    waves of a workgroup add their partial sums through LDS (no atomics: the sum order
+//    is fixed).
+//  * tiled (M > 64, prefill): 128 x 128 x 64 tiles through double-buffered LDS, 4 waves
+//    of 64 x 64, tile order arranged so that the workgroups an XCD runs together share
+//    their W and A tiles in that XCD's L2.
+//
+// Epilogue 1 expects W with gate and up rows interleaved in blocks of 16 and writes
+// silu(gate) * up (llama/model.rs:297-302 of the reference) instead of the two products.
+//
+// Reference loop: y[o] = sum_i W[i + o * n_in] * x[i]  (llama/model.rs:67-91).
+#include "api.h"
+#include "mfma.h"
+
+// =============================================================================== skinny
+template <int MB, int R, int EPI, typename TO>
+__global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
+                                                          const bf16_t* __restrict__ w, TO* __restrict__ c,
+                                                          int m, int n, int k, int k_per_wave) {
+  extern __shared__ float red[];      // [waves - 1][ACC][64]
+  constexpr int ACC = R * MB * 4;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n_waves = blockDim.x >> 6;
+  const int r = lane & 15;
+  const int kq = lane >> 4;
+  const int n0 = blockIdx.x * (16 * R);
+
+  f32x4_t acc[R][MB];
+#pragma unroll
+  for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+    for (int cb = 0; cb < MB; ++cb) acc[rt][cb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  const bf16_t* wrow[R];
+  bool wok[R];
+#pragma unroll
+  for (int rt = 0; rt < R; ++rt) {
+    const int row = n0 + 16 * rt + r;
+    wok[rt] = row < n;
+    wrow[rt] = w + (size_t)(wok[rt] ? row : 0) * k;
+  }
+  const bf16_t* xrow[MB];
+  bool xok[MB];
+#pragma unroll
+  for (int cb = 0; cb < MB; ++cb) {
+    const int row = 16 * cb + r;
+    xok[cb] = row < m;
+    xrow[cb] = x + (size_t)(xok[cb] ? row : 0) * k;
+  }
+
+  const int k_begin = wave * k_per_wave;
+  const int k_end = (k_begin + k_per_wave < k) ? k_begin + k_per_wave : k;
+  for (int k0 = k_begin; k0 < k_end; k0 += 128) {
+    Frag8 a[R][4], b[MB][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int kk = k0 + 32 * j + 8 * kq;
+      const bool in = kk < k_end;
+#pragma unroll
+      for (int rt = 0; rt < R; ++rt) a[rt][j].u = (in && wok[rt]) ? load16(wrow[rt] + kk) : zero16();
+#pragma unroll
+      for (int cb = 0; cb < MB; ++cb) b[cb][j].u = (in && xok[cb]) ? load16(xrow[cb] + kk) : zero16();
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+        for (int cb = 0; cb < MB; ++cb) acc[rt][cb] = mfma16(a[rt][j], b[cb][j], acc[rt][cb]);
+  }
+
+  // ---- partial sums of waves 1.. go through LDS to wave 0
+  if (n_waves > 1) {
+    if (wave > 0) {
+      float* dst = red + (size_t)(wave - 1) * ACC * 64 + lane;
+#pragma unroll
+      for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+        for (int cb = 0; cb < MB; ++cb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dst[((rt * MB + cb) * 4 + i) * 64] = acc[rt][cb][i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+      for (int ww = 0; ww < n_waves - 1; ++ww) {
+        const float* src = red + (size_t)ww * ACC * 64 + lane;
+#pragma unroll
+        for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+          for (int cb = 0; cb < MB; ++cb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[rt][cb][i] += src[((rt * MB + cb) * 4 + i) * 64];
+      }
+    }
+  }
+  if (wave != 0) return;
+
+  // ---- lane holds, per (rt, cb): token 16*cb + r, W rows n0 + 16*rt + 4*kq + 0..3
+  if (EPI == 0) {
+#pragma unroll
+    for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+      for (int cb = 0; cb < MB; ++cb) {
+        const int mm = 16 * cb + r;
+        const int nn = n0 + 16 * rt + 4 * kq;
+        if (mm >= m) continue;
+        TO* dst = c + (size_t)mm * n + nn;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nn + i < n) Num<TO>::store(dst + i, acc[rt][cb][i]);
+      }
+  } else {
+    const int half_n = n / 2;
+#pragma unroll
+    for (int rt = 0; rt + 1 < R; rt += 2)
+#pragma unroll
+      for (int cb = 0; cb < MB; ++cb) {
+        const int mm = 16 * cb + r;
+        const int nn = n0 / 2 + 16 * (rt / 2) + 4 * kq;
+        if (mm >= m) continue;
+        TO* dst = c + (size_t)mm * half_n + nn;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nn + i < half_n) Num<TO>::store(dst + i, silu_f32(acc[rt][cb][i]) * acc[rt + 1][cb][i]);
+      }
+  }
+}
+
+template <int MB, int R, int EPI, typename TO>
+static int launch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
+  int n_waves = k / 256;
+  if (n_waves < 1) n_waves = 1;
+  if (n_waves > 8) n_waves = 8;
+  int k_per_wave = (k + n_waves - 1) / n_waves;
+  k_per_wave = (k_per_wave + 127) / 128 * 128;
+  const size_t lds = (size_t)(n_waves - 1) * R * MB * 4 * 64 * sizeof(float);
+  RB_REQUIRE(lds <= 64 * 1024, "rb_gemm_bf16: internal: reduction buffer of %zu bytes", lds);
+  const int grid = (n + 16 * R - 1) / (16 * R);
+  gemm_skinny_kernel<MB, R, EPI, TO><<<grid, n_waves * 64, lds, s>>>(x, w, (TO*)c, m, n, k, k_per_wave);
+  return 0;
+}
+
+template <int EPI, typename TO>
+static int dispatch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
+  const int mb = (m + 15) / 16;
+  // rows of W per wave: more of them reuse the token operand better, fewer give more
+  // workgroups; keep at least about two workgroups per compute unit
+  int r = 1;
+  if (n >= 32768) r = 4;
+  else if (n >= 16384) r = 2;
+  if (EPI == 1 && r < 2) r = 2;
+  if (mb >= 3 && r > 2) r = 2;
+#define RB_SK(MBV, RV) return launch_skinny<MBV, RV, EPI, TO>(x, w, c, m, n, k, s)
+  if (mb == 1) {
+    if (r == 4) RB_SK(1, 4);
+    if (r == 2) RB_SK(1, 2);
+    if (EPI == 0) RB_SK(1, 1);
+  } else if (mb == 2) {
+    if (r == 4) RB_SK(2, 4);
+    if (r == 2) RB_SK(2, 2);
+    if (EPI == 0) RB_SK(2, 1);
+  } else if (mb == 3) {
+    if (r == 2) RB_SK(3, 2);
+    if (EPI == 0) RB_SK(3, 1);
+  } else {
+    if (r == 2) RB_SK(4, 2);
+    if (EPI == 0) RB_SK(4, 1);
+  }
+#undef RB_SK
+  RB_REQUIRE(false, "rb_gemm_bf16: internal: no skinny kernel for M=%d R=%d", m, r);
+}
+
+// =============================================================================== tiled
+#define TG_BK 64
+#define TG_LD 72          // bf16 elements per LDS row: 64 + 8 of padding, so that the 16 lanes
+                          // of a quarter wave read 16 different 16-byte bank groups
+
+template <int BN, int BM, int WN, int WM, int EPI, typename TO>
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
+                                                         const bf16_t* __restrict__ w, TO* __restrict__ c,
+                                                         int m, int n, int k, int m_tiles, int n_tiles) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int TN = WN / 32, TM = WM / 32;
+  constexpr int WAVES_N = BN / WN;
+  constexpr int W_CHUNKS = BN * 8 / 256, X_CHUNKS = BM * 8 / 256;
+  static_assert((BN / WN) * (BM / WM) == 4, "four waves");
+  bf16_t* ws = reinterpret_cast<bf16_t*>(smem);                      // [2][BN][TG_LD]
+  bf16_t* xs = ws + 2 * BN * TG_LD;                                  // [2][BM][TG_LD]
+
+  // tile order: workgroup ids go round robin over the 8 XCDs; give each XCD a contiguous
+  // range of tiles, tokens fastest, so that what it runs together shares W and A tiles
+  const int tiles = m_tiles * n_tiles;
+  const int per_xcd = (tiles + 7) / 8;
+  const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (t >= tiles) return;
+  const int m0 = (t % m_tiles) * BM;
+  const int n0 = (t / m_tiles) * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wn0 = (wave % WAVES_N) * WN;
+  const int wm0 = (wave / WAVES_N) * WM;
+  const int l32 = lane & 31;
+  const int g = lane >> 5;
+
+  f32x16_t acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  uint4 wreg[W_CHUNKS], xreg[X_CHUNKS];
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < W_CHUNKS; ++i) {
+      const int q = tid + 256 * i;
+      const int row = n0 + q / 8, kk = k0 + (q % 8) * 8;
+      wreg[i] = (row < n && kk < k) ? load16(w + (size_t)row * k + kk) : zero16();
+    }
+#pragma unroll
+    for (int i = 0; i < X_CHUNKS; ++i) {
+      const int q = tid + 256 * i;
+      const int row = m0 + q / 8, kk = k0 + (q % 8) * 8;
+      xreg[i] = (row < m && kk < k) ? load16(x + (size_t)row * k + kk) : zero16();
+    }
+  };
+  auto store_lds = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < W_CHUNKS; ++i) {
+      const int q = tid + 256 * i;
+      *reinterpret_cast<uint4*>(ws + ((size_t)buf * BN + q / 8) * TG_LD + (q % 8) * 8) = wreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < X_CHUNKS; ++i) {
+      const int q = tid + 256 * i;
+      *reinterpret_cast<uint4*>(xs + ((size_t)buf * BM + q / 8) * TG_LD + (q % 8) * 8) = xreg[i];
+    }
+  };
+
+  const int k_tiles = (k + TG_BK - 1) / TG_BK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < k_tiles) load_global((kt + 1) * TG_BK);
+    const bf16_t* wb = ws + (size_t)buf * BN * TG_LD;
+    const bf16_t* xb = xs + (size_t)buf * BM * TG_LD;
+#pragma unroll
+    for (int ks = 0; ks < TG_BK / 16; ++ks) {
+      Frag8 a[TN], b[TM];
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+        a[i].u = *reinterpret_cast<const uint4*>(wb + (size_t)(wn0 + 32 * i + l32) * TG_LD + ks * 16 + g * 8);
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+        b[j].u = *reinterpret_cast<const uint4*>(xb + (size_t)(wm0 + 32 * j + l32) * TG_LD + ks * 16 + g * 8);
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+    }
+    if (kt + 1 < k_tiles) store_lds(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- lane holds, per (i, j): token m0 + wm0 + 32 j + l32, W rows base + 8 (e / 4) + 4 g + e % 4
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int mm = m0 + wm0 + 32 * j + l32;
+      if (mm >= m) continue;
+      const int nbase = n0 + wn0 + 32 * i;
+      if (EPI == 0) {
+        TO* dst = c + (size_t)mm * n;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int nn = nbase + 8 * (e / 4) + 4 * g + (e % 4);
+          if (nn < n) Num<TO>::store(dst + nn, acc[i][j][e]);
+        }
+      } else {
+        const int half_n = n / 2;
+        TO* dst = c + (size_t)mm * half_n;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int nn = nbase / 2 + 8 * (e / 4) + 4 * g + (e % 4);
+          if (nn < half_n) Num<TO>::store(dst + nn, silu_f32(acc[i][j][e]) * acc[i][j][e + 8]);
+        }
+      }
+    }
+}
+
+template <int EPI, typename TO>
+static int launch_tiled(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
+  constexpr int BN = 128, BM = 128;
+  const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
+  const long long tiles = (long long)m_tiles * n_tiles;
+  RB_REQUIRE(tiles < (1LL << 30), "rb_gemm_bf16: too many tiles");
+  const size_t lds = (size_t)2 * (BN + BM) * TG_LD * sizeof(bf16_t);
+  auto kern = gemm_tiled_kernel<BN, BM, 64, 64, EPI, TO>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    RB_REQUIRE(e == hipSuccess, "rb_gemm_bf16: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    configured = true;
+  }
+  const int grid = (int)((tiles + 7) / 8 * 8);
+  kern<<<grid, 256, lds, s>>>(x, w, (TO*)c, m, n, k, m_tiles, n_tiles);
+  return 0;
+}
+
+extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out, int epilogue, int m, int n,
+                            int k, void* stream) {
+  RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_bf16: bad sizes M=%d N=%d K=%d", m, n, k);
+  RB_REQUIRE(k % 8 == 0, "rb_gemm_bf16: K=%d must be a multiple of 8 (use rb_gemm_generic)", k);
+  RB_REQUIRE(epilogue == 0 || epilogue == 1, "rb_gemm_bf16: unknown epilogue %d", epilogue);
+  RB_REQUIRE(epilogue == 0 || n % 32 == 0, "rb_gemm_bf16: gated epilogue needs N=%d to be a multiple of 32", n);
+  RB_REQUIRE(dtype_out == RB_F32 || dtype_out == RB_BF16, "rb_gemm_bf16: unknown output dtype %d", dtype_out);
+  if (m == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const bf16_t* xa = (const bf16_t*)a;
+  const bf16_t* wa = (const bf16_t*)w;
+  int rc;
+  if (m <= 64) {
+    if (epilogue == 0)
+      rc = dtype_out == RB_F32 ? dispatch_skinny<0, float>(xa, wa, c, m, n, k, s)
+                               : dispatch_skinny<0, bf16_t>(xa, wa, c, m, n, k, s);
+    else
+      rc = dtype_out == RB_F32 ? dispatch_skinny<1, float>(xa, wa, c, m, n, k, s)
+                               : dispatch_skinny<1, bf16_t>(xa, wa, c, m, n, k, s);
+  } else {
+    if (epilogue == 0)
+      rc = dtype_out == RB_F32 ? launch_tiled<0, float>(xa, wa, c, m, n, k, s)
+                               : launch_tiled<0, bf16_t>(xa, wa, c, m, n, k, s);
+    else
+      rc = dtype_out == RB_F32 ? launch_tiled<1, float>(xa, wa, c, m, n, k, s)
+                               : launch_tiled<1, bf16_t>(xa, wa, c, m, n, k, s);
+  }
+  if (rc) return rc;
+  RB_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,239 @@
+"""ctypes binding of librbitnet_hip.so: torch tensors in, kernels launched on torch's
+current HIP stream.  There is no fallback: without a GPU and the built library every
+call fails with a KernelError."""
+from __future__ import annotations
+
+import ctypes
+import threading
+from typing import Optional
+
+import torch
+
+from ..errors import KernelError
+from . import build as _build
+
+_F32, _BF16 = 0, 1
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_F = ctypes.c_float
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _F32
+    if dtype == torch.bfloat16:
+        return _BF16
+    raise KernelError(f"the kernels take float32 or bfloat16 storage, not {dtype}")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    if t is None:
+        return None
+    return t.data_ptr()
+
+
+def _check(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    if not t.is_cuda:
+        raise KernelError(f"{name} must be on the GPU")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, found {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name} must have shape {tuple(shape)}, found {tuple(t.shape)}")
+
+
+class Kernels:
+    """The loaded library.  Methods check operand shapes on the host before a launch, so
+    that a kernel never sees sizes other than the ones its grid assumes."""
+
+    def __init__(self, path: Optional[str] = None):
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU visible: rbitnet_amd runs on an MI355X (gfx950) only and has no CPU fallback")
+        path = path or _build.ensure_built()
+        try:
+            self._lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError(f"cannot load the HIP kernel library {path}: {e}") from None
+        self.path = path
+        L = self._lib
+        L.rb_last_error.restype = ctypes.c_char_p
+        sig = {
+            "rb_embed_gather": [_P, _I, _P, _P, _I, _I, _P],
+            "rb_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _I, _P, _I, _P],
+            "rb_rope_kv_write": [_P, _P, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "rb_swiglu": [_P, _P, _I, _I, _I, _P],
+            "rb_gemm_generic": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "rb_gemm_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "rb_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
+            "rb_attention_prefill_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+            "rb_attention_decode_bf16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
+            "rb_sample": [_P, _I, _I, _P, _P, _P, _P],
+        }
+        for name, args in sig.items():
+            fn = getattr(L, name)
+            fn.argtypes = args
+            fn.restype = _I
+        self.page_size = int(L.rb_page_size())
+
+    # ------------------------------------------------------------------ helpers
+    @staticmethod
+    def _stream() -> int:
+        return torch.cuda.current_stream().cuda_stream
+
+    def _ok(self, rc: int) -> None:
+        if rc != 0:
+            raise KernelError(self._lib.rb_last_error().decode("utf-8", "replace"))
+
+    # ------------------------------------------------------------------ ops
+    def embed_gather(self, table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+        n, width = out.shape
+        _check(table, "table")
+        _check(ids, "ids", torch.int32, (n,))
+        _check(out, "out", torch.float32)
+        if table.shape[1] != width:
+            raise KernelError("embedding width mismatch")
+        self._ok(self._lib.rb_embed_gather(_ptr(table), dtype_code(table.dtype), _ptr(ids), _ptr(out), n, width,
+                                           self._stream()))
+
+    def add_rmsnorm(self, x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, eps: float,
+                    rows: Optional[torch.Tensor], out: torch.Tensor) -> None:
+        n_rows, width = out.shape
+        _check(x, "x", torch.float32)
+        if x.shape[1] != width:
+            raise KernelError("norm width mismatch")
+        if delta is not None:
+            _check(delta, "delta", torch.float32, x.shape)
+        _check(gain, "gain", torch.float32, (width,))
+        if rows is not None:
+            _check(rows, "rows", torch.int32, (n_rows,))
+        elif x.shape[0] != n_rows:
+            raise KernelError("norm row count mismatch")
+        _check(out, "out")
+        self._ok(self._lib.rb_add_rmsnorm(_ptr(x), _ptr(delta), _ptr(gain), float(eps), _ptr(rows), n_rows, width,
+                                          _ptr(out), dtype_code(out.dtype), self._stream()))
+
+    def rope_kv_write(self, qkv, cos, sin, style, q_out, k_pages, v_pages, tok_pos, tok_seq, block_table,
+                      n_heads, n_kv, head_dim) -> None:
+        n = qkv.shape[0]
+        _check(qkv, "qkv", torch.float32, (n, (n_heads + 2 * n_kv) * head_dim))
+        _check(q_out, "q_out", None, (n, n_heads, head_dim))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(tok_seq, "tok_seq", torch.int32, (n,))
+        _check(block_table, "block_table", torch.int32)
+        if cos is not None:
+            _check(cos, "cos", torch.float32)
+            _check(sin, "sin", torch.float32, cos.shape)
+            if cos.shape[1] != head_dim // 2:
+                raise KernelError("angle table width mismatch")
+        if k_pages is not None:
+            _check(k_pages, "k_pages", q_out.dtype)
+            _check(v_pages, "v_pages", q_out.dtype, k_pages.shape)
+            if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, head_dim):
+                raise KernelError(f"cache pages have shape {tuple(k_pages.shape)}, expected "
+                                  f"[*, {n_kv}, {self.page_size}, {head_dim}]")
+        self._ok(self._lib.rb_rope_kv_write(_ptr(qkv), _ptr(cos), _ptr(sin), int(style), _ptr(q_out), _ptr(k_pages),
+                                            _ptr(v_pages), dtype_code(q_out.dtype), _ptr(tok_pos), _ptr(tok_seq),
+                                            _ptr(block_table), block_table.shape[1], n, n_heads, n_kv, head_dim,
+                                            self._stream()))
+
+    def swiglu(self, gu: torch.Tensor, out: torch.Tensor) -> None:
+        n, ff = out.shape
+        _check(gu, "gu", torch.float32, (n, 2 * ff))
+        _check(out, "out")
+        self._ok(self._lib.rb_swiglu(_ptr(gu), _ptr(out), dtype_code(out.dtype), n, ff, self._stream()))
+
+    def gemm_generic(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor) -> None:
+        m, k = a.shape
+        n = w.shape[0]
+        _check(a, "a")
+        _check(w, "w", a.dtype, (n, k))
+        _check(c, "c", None, (m, n))
+        self._ok(self._lib.rb_gemm_generic(_ptr(a), _ptr(w), _ptr(c), dtype_code(a.dtype), dtype_code(c.dtype),
+                                           m, n, k, self._stream()))
+
+    def gemm_bf16(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = 0) -> None:
+        m, k = a.shape
+        n = w.shape[0]
+        _check(a, "a", torch.bfloat16)
+        _check(w, "w", torch.bfloat16, (n, k))
+        _check(c, "c", None, (m, n // 2 if epilogue == 1 else n))
+        self._ok(self._lib.rb_gemm_bf16(_ptr(a), _ptr(w), _ptr(c), dtype_code(c.dtype), int(epilogue), m, n, k,
+                                        self._stream()))
+
+    def attention_generic(self, q, k_pages, v_pages, out, tok_pos, tok_seq, block_table, n_heads, n_kv, head_dim,
+                          scale, window) -> None:
+        n = q.shape[0]
+        _check(q, "q", None, (n, n_heads, head_dim))
+        _check(k_pages, "k_pages", q.dtype)
+        _check(v_pages, "v_pages", q.dtype, k_pages.shape)
+        if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, head_dim):
+            raise KernelError("cache pages do not match the head counts")
+        _check(out, "out", q.dtype, (n, n_heads * head_dim))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(tok_seq, "tok_seq", torch.int32, (n,))
+        _check(block_table, "block_table", torch.int32)
+        self._ok(self._lib.rb_attention_generic(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), dtype_code(q.dtype),
+                                                _ptr(tok_pos), _ptr(tok_seq), _ptr(block_table),
+                                                block_table.shape[1], n, n_heads, n_kv, head_dim, float(scale),
+                                                int(window or 0), self._stream()))
+
+    def attention_prefill_bf16(self, q, k_pages, v_pages, out, cu_seqlens, past_len, block_table, n_seqs,
+                               max_q_len, n_heads, n_kv, head_dim, scale, window) -> None:
+        n = q.shape[0]
+        _check(q, "q", torch.bfloat16, (n, n_heads, head_dim))
+        _check(k_pages, "k_pages", torch.bfloat16)
+        _check(v_pages, "v_pages", torch.bfloat16, k_pages.shape)
+        if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, head_dim):
+            raise KernelError("cache pages do not match the head counts")
+        _check(out, "out", torch.bfloat16, (n, n_heads * head_dim))
+        _check(cu_seqlens, "cu_seqlens", torch.int32, (n_seqs + 1,))
+        _check(past_len, "past_len", torch.int32, (n_seqs,))
+        _check(block_table, "block_table", torch.int32)
+        self._ok(self._lib.rb_attention_prefill_bf16(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out),
+                                                     _ptr(cu_seqlens), _ptr(past_len), _ptr(block_table),
+                                                     block_table.shape[1], n_seqs, int(max_q_len), n_heads, n_kv,
+                                                     head_dim, float(scale), int(window or 0), self._stream()))
+
+    def attention_decode_bf16(self, q, k_pages, v_pages, out, tok_pos, block_table, n_heads, n_kv, head_dim,
+                              scale, window, n_splits, workspace) -> None:
+        n = q.shape[0]
+        _check(q, "q", torch.bfloat16, (n, n_heads, head_dim))
+        _check(k_pages, "k_pages", torch.bfloat16)
+        _check(v_pages, "v_pages", torch.bfloat16, k_pages.shape)
+        if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, head_dim):
+            raise KernelError("cache pages do not match the head counts")
+        _check(out, "out", torch.bfloat16, (n, n_heads * head_dim))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(block_table, "block_table", torch.int32)
+        _check(workspace, "workspace", torch.float32)
+        if workspace.numel() < n * n_heads * n_splits * (head_dim + 2):
+            raise KernelError("decode attention workspace too small")
+        self._ok(self._lib.rb_attention_decode_bf16(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tok_pos),
+                                                    _ptr(block_table), block_table.shape[1], n, n_heads, n_kv,
+                                                    head_dim, float(scale), int(window or 0), int(n_splits),
+                                                    _ptr(workspace), self._stream()))
+
+    def sample(self, logits: torch.Tensor, temperature: Optional[torch.Tensor], u: Optional[torch.Tensor],
+               tokens: torch.Tensor) -> None:
+        n, vocab = logits.shape
+        _check(logits, "logits", torch.float32)
+        if temperature is not None:
+            _check(temperature, "temperature", torch.float32, (n,))
+            _check(u, "u", torch.float32, (n,))
+        _check(tokens, "tokens", torch.int32, (n,))
+        self._ok(self._lib.rb_sample(_ptr(logits), n, vocab, _ptr(temperature), _ptr(u), _ptr(tokens),
+                                     self._stream()))
+
+
+_lock = threading.Lock()
+_instance: Optional[Kernels] = None
+
+
+def kernels() -> Kernels:
+    """The process-wide library, loaded (and built, if it is not) at first use."""
+    global _instance
+    with _lock:
+        if _instance is None:
+            _instance = Kernels()
+        return _instance

@@ -1,0 +1,35 @@
+// Matrix-core (MFMA) operand types and layouts for gfx950, wave of 64 lanes.
+//
+// v_mfma_f32_16x16x32_bf16: D[16 x 16] += A[16 x 32] * B[32 x 16]
+//   A: lane l holds row l % 16, the 8 depth values of group l / 16
+//   B: lane l holds column l % 16, the 8 depth values of group l / 16
+//   D: lane l holds column l % 16, rows 4 * (l / 16) + i for i = 0..3
+// v_mfma_f32_32x32x16_bf16: D[32 x 32] += A[32 x 16] * B[16 x 32]
+//   A: lane l holds row l % 32, the 8 depth values of group l / 32
+//   B: lane l holds column l % 32, the 8 depth values of group l / 32
+//   D: lane l holds column l % 32, rows 8 * (i / 4) + 4 * (l / 32) + i % 4 for i = 0..15
+// Which depth values a group holds is free as long as A and B agree, since the product
+// sums over them.
+#pragma once
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+union Frag8 {
+  uint4 u;
+  bf16x8_t v;
+};
+
+__device__ __forceinline__ f32x4_t mfma16(const Frag8& a, const Frag8& b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x16_t mfma32(const Frag8& a, const Frag8& b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ uint4 load16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ uint4 zero16() { return make_uint4(0u, 0u, 0u, 0u); }
+
+__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + expf(-v)); }

@@ -1,0 +1,172 @@
+"""The engine: a model, its cache and ONE step function.
+
+The reference's engine (crates/bitnet-core/src/inference.rs:74-209) owns one runtime
+with one sequence and feeds it a token at a time (llama/runtime.rs:50-53,
+llama/model.rs:219).  This one serves a batch of sequences that start together with
+unequal lengths: `step` takes, per sequence, the tokens to run next (a whole prompt,
+a piece of it, or one decoded token), runs exactly those as one packed batch on top of
+what the cache holds, and returns float32 logits at the asked places only.
+
+Guards as in model.rs:221-227: a token id outside the vocabulary and a position beyond
+the model's or the cache's limit are errors raised before anything is launched.
+"""
+from __future__ import annotations
+
+import os
+from typing import Any, Dict, List, Optional, Sequence, Tuple, Union
+
+import torch
+
+from ..cache import PAGE_SIZE, Cache, pages_for
+from ..config import load_config
+from ..errors import CacheError, ConfigError, InferenceError, KernelError
+from ..weights import DEFAULT_SEED, load_weights, random_tensors
+from .context import StepContext
+from .model import Model
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def parse_dtype(dtype: Any) -> torch.dtype:
+    if dtype not in _DTYPES:
+        raise ConfigError(f"dtype must be 'bfloat16' or 'float32', found {dtype!r}")
+    return _DTYPES[dtype]
+
+
+class Engine:
+    def __init__(self, config: Any, spec, model: Model, max_tokens: int, max_batch: int,
+                 max_seq_len: Optional[int] = None):
+        self.config = config
+        self.spec = spec
+        self.model = model
+        self.lib = model.lib
+        self.device = model.device
+        self.dtype = model.dtype
+        self.max_seq_len = min(int(max_seq_len or spec.max_positions), spec.max_positions)
+        self.max_batch = int(max_batch)
+        self.cache = Cache(model.cache_requests(), n_slots=self.max_batch, max_tokens=max_tokens,
+                           dtype=self.dtype, device=self.device, readers=model.cache_readers())
+        self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0}
+        from ..sampling import Sampler
+        self.sampler = Sampler(self.lib, self.device)
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def _build(cls, config_source: Any, tensors_for, dtype: Any, max_tokens: Optional[int], max_batch: Optional[int],
+               max_seq_len: Optional[int], device: str, generic_only: bool) -> "Engine":
+        from ..csrc.lib import kernels
+        cfg, spec = load_config(config_source)
+        lib = kernels()                       # raises when there is no GPU or no built library
+        tdtype = parse_dtype(dtype)
+        model = Model(spec, tdtype, device, lib, generic_only=generic_only)
+        model.load(tensors_for(model, cfg))
+        seq = min(int(max_seq_len or spec.max_positions), spec.max_positions)
+        if max_batch is None:
+            max_batch = 8 if max_tokens is None else max(1, min(pages_for(max_tokens), 1024))
+        if max_tokens is None:
+            max_tokens = max_batch * pages_for(seq) * PAGE_SIZE
+        return cls(cfg, spec, model, max_tokens=max_tokens, max_batch=max_batch, max_seq_len=seq)
+
+    @classmethod
+    def load_path(cls, path: str, dtype: Any = "bfloat16", max_tokens: Optional[int] = None,
+                  max_batch: Optional[int] = None, max_seq_len: Optional[int] = None, device: str = "cuda:0",
+                  generic_only: bool = False) -> "Engine":
+        """A model folder (config.json + model.safetensors), as the reference's
+        `Engine::load_path` takes a GGUF path (inference.rs:121-133)."""
+        def tensors_for(model: Model, cfg):
+            aliases = getattr(type(cfg), "tensor_aliases", None)
+            ignored = ["lm_head.weight"] if model.spec.head_name is None else []
+            return load_weights(path, model.expected, aliases=aliases, ignored=ignored)
+
+        return cls._build(path, tensors_for, dtype, max_tokens, max_batch, max_seq_len, device, generic_only)
+
+    @classmethod
+    def random(cls, config: Any, seed: int = DEFAULT_SEED, dtype: Any = "bfloat16", std: float = 0.02,
+               norm_std: float = 0.02, max_tokens: Optional[int] = None, max_batch: Optional[int] = None,
+               max_seq_len: Optional[int] = None, device: str = "cuda:0", generic_only: bool = False) -> "Engine":
+        """Random weights drawn on the GPU from a configuration and a seed, no files: the
+        counterpart of the reference's toy mode (RBITNET_TOY / RBITNET_TOY_SEED,
+        inference.rs:24-36)."""
+        def tensors_for(model: Model, cfg):
+            store = torch.bfloat16 if model.dtype == torch.bfloat16 else torch.float32
+            return dict(random_tensors(model.expected, seed, std, norm_std, store, device))
+
+        return cls._build(config, tensors_for, dtype, max_tokens, max_batch, max_seq_len, device, generic_only)
+
+    # ------------------------------------------------------------------ slots
+    def alloc_slot(self) -> int:
+        return self.cache.alloc_slot()
+
+    def free_slot(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    def room(self, slot: int) -> int:
+        """How many more tokens the sequence may hold (model and engine limits)."""
+        return self.max_seq_len - self.cache.length(slot)
+
+    # ------------------------------------------------------------------ the step
+    def step(self, entries: Sequence[Tuple[int, Sequence[int]]],
+             want: Union[str, Sequence[Sequence[int]]] = "last") -> torch.Tensor:
+        """entries: (slot, tokens to run next) per sequence, at least one token each.
+        want: "last" (the last token of each entry), "all", or per entry the indices
+        among its tokens whose logits are asked for (may be empty).
+        Returns float32 [number of asked places, vocab], in the order of entries and want."""
+        if not entries:
+            raise InferenceError("a step needs at least one sequence")
+        slots = [int(s) for s, _ in entries]
+        tokens = [list(t) for _, t in entries]
+        vocab = self.spec.vocab_size
+        past = []
+        for s, toks in zip(slots, tokens):
+            if not toks:
+                raise InferenceError(f"slot {s}: a step brings at least one token per sequence")
+            n = self.cache.length(s)
+            if n + len(toks) > self.max_seq_len:
+                raise InferenceError(
+                    f"slot {s}: sequence position >= max_seq ({n} + {len(toks)} tokens exceed {self.max_seq_len})")
+            for t in toks:
+                if not 0 <= int(t) < vocab:
+                    raise InferenceError(f"slot {s}: token id out of range ({t}, vocabulary {vocab})")
+            past.append(n)
+        rows: List[int] = []
+        base = 0
+        for i, toks in enumerate(tokens):
+            if want == "last":
+                idx = [len(toks) - 1]
+            elif want == "all":
+                idx = range(len(toks))
+            else:
+                idx = want[i]
+            for j in idx:
+                if not 0 <= int(j) < len(toks):
+                    raise InferenceError(f"slot {slots[i]}: wanted place {j} is not among its {len(toks)} tokens")
+                rows.append(base + int(j))
+            base += len(toks)
+        q_lens = [len(t) for t in tokens]
+        self.cache.reserve(slots, q_lens)
+        tables = {id(g): self.cache.block_table(g, slots) for g in self.cache.kv_groups}
+        ctx = StepContext(self.device, slots, past, tokens, rows, tables)
+        logits = self.model.forward(ctx, self.cache, ctx.rows)
+        self.cache.commit(slots, q_lens)
+        self.stats["steps"] += 1
+        if max(q_lens) == 1:
+            self.stats["decode_tokens"] += len(slots)
+        else:
+            self.stats["prefill_tokens"] += sum(q_lens)
+        return logits
+
+    # ------------------------------------------------------------------ generation
+    def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 256, temperature: float = 0.7,
+                 seed: int = 0, stop_token_ids: Optional[Sequence[int]] = None):
+        from .generate import generate
+        return generate(self, prompts, max_tokens=max_tokens, temperature=temperature, seed=seed,
+                        stop_token_ids=stop_token_ids)
+
+    def complete(self, prompt: Sequence[int], max_tokens: int = 256, temperature: float = 0.7, seed: int = 0):
+        """One prompt in, its new tokens out: `Engine::complete(prompt, max_tokens,
+        temperature)` of the reference (inference.rs:183) on token ids."""
+        return self.generate([prompt], max_tokens=max_tokens, temperature=temperature, seed=seed)[0].tokens

@@ -1,0 +1,112 @@
+"""The attention mixer: grouped-query causal attention over the paged cache.
+
+Reference, one token (crates/bitnet-core/src/llama/model.rs:238-294): q = Wq h, k = Wk h,
+v = Wv h; rotate every q head and k head; store k (rotated) and v at the token's
+position; for q head qh read kv head qh / (Hq / Hk); scores (q . k) * scale over the
+keys up to the token's own position; softmax; weighted sum of v; heads concatenated;
+out = Wo attn.  Here the same runs for all tokens of a step at once: keys and values
+of the whole step are written to the cache first, then every token attends to the
+cache up to its own position, so a step may bring any number of tokens per sequence
+on top of any past.
+
+Parameters: num_heads, num_kv_heads, head_dim, scale, window (None: all keys; n: the
+last n keys including the token's own), position (a PartSpec), cache_from (None, or the
+index of the layer whose cache this layer reads instead of keeping one), names (tensor
+names of the four matrices relative to the layer's prefix).
+
+Interface of a mixer:
+  tensor_specs() / load(tensors)
+  cache_request() -> CacheRequest or None
+  forward(h [T, E] compute dtype, ctx, view) -> float32 [T, E]
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..errors import ConfigError, KernelError
+from .base import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register_mixer
+from .linear import linear
+
+DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight"}
+_MATRIX_CORE_HEAD_DIMS = (64, 128)
+
+
+class Attention(Part):
+    def __init__(self, params: Dict, env: BuildEnv):
+        self.env = env
+        self.n_heads = int(params["num_heads"])
+        self.n_kv = int(params["num_kv_heads"])
+        self.head_dim = int(params["head_dim"])
+        if self.n_heads <= 0 or self.n_kv <= 0 or self.n_heads % self.n_kv != 0:
+            raise ConfigError(f"attention: {self.n_heads} heads cannot share {self.n_kv} kv heads")
+        if self.head_dim <= 0 or self.head_dim % 2 != 0 or self.head_dim > 256:
+            raise ConfigError(f"attention: head_dim {self.head_dim} not supported (even, at most 256)")
+        self.scale = float(params.get("scale") or self.head_dim ** -0.5)
+        self.window = params.get("window")
+        if self.window is not None and int(self.window) <= 0:
+            raise ConfigError("attention: window must be positive")
+        self.cache_from = params.get("cache_from")
+        self.names = dict(DEFAULT_NAMES, **(params.get("names") or {}))
+        self.position = build_part("position", params["position"], env)
+        self.hidden = env.hidden_size
+        self.w_qkv: Optional[torch.Tensor] = None
+        self.w_q: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+
+    # ------------------------------------------------------------------ tensors
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        qd, kd = self.n_heads * self.head_dim, self.n_kv * self.head_dim
+        specs = {self.names["q"]: TensorSpec((qd, self.hidden)), self.names["o"]: TensorSpec((self.hidden, qd))}
+        if self.cache_from is None:
+            specs[self.names["k"]] = TensorSpec((kd, self.hidden))
+            specs[self.names["v"]] = TensorSpec((kd, self.hidden))
+        return specs
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        # q, k and v rows in one matrix: one product per step instead of three
+        if self.cache_from is None:
+            self.w_qkv = torch.cat([tensors[self.names["q"]], tensors[self.names["k"]],
+                                    tensors[self.names["v"]]], dim=0).contiguous()
+        else:
+            self.w_qkv = tensors[self.names["q"]].contiguous()
+        self.w_o = tensors[self.names["o"]].contiguous()
+
+    def cache_request(self) -> Optional[CacheRequest]:
+        if self.cache_from is not None:
+            return None
+        return CacheRequest("kv", heads=self.n_kv, head_dim=self.head_dim,
+                            window=None if self.window is None else int(self.window))
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, h: torch.Tensor, ctx, view) -> torch.Tensor:
+        lib = self.env.lib
+        t = h.shape[0]
+        hq, hk, d = self.n_heads, self.n_kv, self.head_dim
+        owns = self.cache_from is None
+        qkv = linear(lib, h, self.w_qkv, torch.float32)
+        q = torch.empty((t, hq, d), dtype=self.env.dtype, device=h.device)
+        bt = view.block_table
+        if owns:
+            self.position.encode_and_store(qkv, q, view.k_pages, view.v_pages, ctx, bt, hq, hk, d)
+        else:
+            self.position.encode_and_store(qkv, q, None, None, ctx, bt, hq, 0, d)
+        attn = torch.empty((t, hq * d), dtype=self.env.dtype, device=h.device)
+        window = int(self.window) if self.window is not None else 0
+        fast = (self.env.dtype == torch.bfloat16 and d in _MATRIX_CORE_HEAD_DIMS
+                and not getattr(self.env, "generic_only", False))
+        if fast and ctx.max_q_len == 1:
+            n_splits, workspace = ctx.decode_workspace(hq, d)
+            lib.attention_decode_bf16(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, bt, hq, hk, d,
+                                      self.scale, window, n_splits, workspace)
+        elif fast:
+            lib.attention_prefill_bf16(q, view.k_pages, view.v_pages, attn, ctx.cu_seqlens, ctx.past_len, bt,
+                                       ctx.n_seqs, ctx.max_q_len, hq, hk, d, self.scale, window)
+        else:
+            lib.attention_generic(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, bt, hq, hk, d,
+                                  self.scale, window)
+        return linear(lib, attn, self.w_o, torch.float32)
+
+
+register_mixer("attention", Attention)

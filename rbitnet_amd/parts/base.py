@@ -1,0 +1,119 @@
+"""What every part is: a kind name, parameters, tensors it owns, a forward.
+
+Kinds of parts and the registry each lives in:
+
+* norm            `register_norm`           forward(x_f32 [T, E], delta, rows) -> h [rows, E]
+* position        `register_position`       a table or rule keyed by absolute position
+* mixer           `register_mixer`          forward(h [T, E], ctx, view) -> [T, E_out]
+* feed-forward    `register_feed_forward`   forward(h [T, E], ctx) -> [T, E]
+* block           `register_block`          arranges norm, mixer, norm, feed-forward
+
+A part is built from `(params, env)`: `params` is the dict of its `PartSpec`,
+`env` a `BuildEnv` (model width, compute dtype, device, the kernel library).
+It declares its tensors (`tensor_specs`) with names relative to its own prefix,
+and receives them in `load`.  A mixer further declares what it needs of the
+cache (`cache_request`).  No part sees the configuration it came from or the
+model it is in.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, Optional, Tuple
+
+import torch
+
+from ..errors import ConfigError
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """A tensor a part owns.
+
+    role "matrix": held in the compute dtype (bfloat16 or float32);
+    role "gain":   a norm's gain, held in float32 (widening is exact);
+    role "table":  integers, held as int32.
+    init names the random initialisation: "normal" is N(0, std), "ones_normal"
+    is 1 + N(0, norm_std)."""
+    shape: Tuple[int, ...]
+    role: str = "matrix"
+    init: str = "normal"
+
+
+@dataclass
+class BuildEnv:
+    hidden_size: int
+    dtype: torch.dtype
+    device: torch.device
+    lib: Any                    # rbitnet_amd.csrc.lib.Kernels (None when only shapes are wanted)
+    layer_index: int = -1
+
+
+@dataclass
+class CacheRequest:
+    """What a mixer needs of the cache.
+
+    kind "kv":    keys and values per token, `heads` x `head_dim` each; `window`
+                  (None = all) is how far back a query looks, so that pages
+                  behind it can be given back.
+    kind "state": `state_shape` numbers per sequence, set to `state_init` when a
+                  slot is handed out.
+    Layers with equal requests share one group of storage."""
+    kind: str
+    heads: int = 0
+    head_dim: int = 0
+    window: Optional[int] = None
+    state_shape: Tuple[int, ...] = ()
+    state_init: float = 0.0
+    state_dtype: torch.dtype = torch.float32
+
+    def key(self) -> Tuple:
+        return (self.kind, self.heads, self.head_dim, self.window, tuple(self.state_shape),
+                self.state_init, self.state_dtype)
+
+
+class Part:
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        pass
+
+
+_REGISTRIES: Dict[str, Dict[str, Callable[..., Any]]] = {
+    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {},
+}
+
+
+def _register(group: str, kind: str, factory: Callable[..., Any]) -> None:
+    _REGISTRIES[group][kind] = factory
+
+
+def register_norm(kind: str, factory: Callable[..., Any]) -> None:
+    _register("norm", kind, factory)
+
+
+def register_position(kind: str, factory: Callable[..., Any]) -> None:
+    _register("position", kind, factory)
+
+
+def register_mixer(kind: str, factory: Callable[..., Any]) -> None:
+    _register("mixer", kind, factory)
+
+
+def register_feed_forward(kind: str, factory: Callable[..., Any]) -> None:
+    _register("feed_forward", kind, factory)
+
+
+def register_block(kind: str, factory: Callable[..., Any]) -> None:
+    _register("block", kind, factory)
+
+
+def build_part(group: str, spec: Any, env: BuildEnv) -> Any:
+    table = _REGISTRIES[group]
+    if spec.kind not in table:
+        raise ConfigError(f"unknown {group} kind {spec.kind!r}; registered: {', '.join(sorted(table))}")
+    return table[spec.kind](spec.params, env)
+
+
+def registered(group: str):
+    return sorted(_REGISTRIES[group])

@@ -1,0 +1,44 @@
+"""How the parts of one layer are arranged.
+
+"prenorm" (crates/bitnet-core/src/llama/model.rs:236-307):
+    x += mixer(norm1(x));  x += feed_forward(norm2(x))
+The residual stream x is float32 and each sum is done by the norm that follows it (see
+norm.py), so a block takes the previous block's not yet added output as `pending` and
+returns its own.  The model adds the last one in the final norm.
+
+Interface of a block: parts() -> {name: part} for the loader (names are tensor-name
+segments below the layer's prefix); mixer (for the cache request);
+forward(x, pending, ctx, view) -> pending.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .base import BuildEnv, build_part, register_block
+
+DEFAULT_SEGMENTS = {"norm1": "input_layernorm", "mixer": "self_attn", "norm2": "post_attention_layernorm",
+                    "feed_forward": "mlp"}
+
+
+class PreNormBlock:
+    def __init__(self, layer_spec, env: BuildEnv):
+        self.norm1 = build_part("norm", layer_spec.norm1, env)
+        self.mixer = build_part("mixer", layer_spec.mixer, env)
+        self.norm2 = build_part("norm", layer_spec.norm2, env)
+        self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, env)
+        self.segments = dict(DEFAULT_SEGMENTS, **(getattr(layer_spec, "segments", None) or {}))
+
+    def parts(self) -> Dict[str, object]:
+        return {self.segments["norm1"]: self.norm1, self.segments["mixer"]: self.mixer,
+                self.segments["norm2"]: self.norm2, self.segments["feed_forward"]: self.feed_forward}
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx, view) -> torch.Tensor:
+        h = self.norm1.forward(x, pending)
+        a = self.mixer.forward(h, ctx, view)
+        h2 = self.norm2.forward(x, a)
+        return self.feed_forward.forward(h2, ctx)
+
+
+register_block("prenorm", PreNormBlock)

@@ -1,0 +1,86 @@
+"""Tiny configurations, model folders and oracle logits shared by the tests."""
+from __future__ import annotations
+
+import json
+import os
+import tempfile
+from functools import lru_cache
+
+import numpy as np
+import torch
+
+# Two tiny Llama configurations that differ in every size and option, and a third whose
+# sizes let the bfloat16 path take its matrix-core kernels (head size 64, widths that are
+# multiples of 16, head_dim given explicitly and not hidden / heads).
+TINY_A = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 64, "num_hidden_layers": 2,
+    "num_attention_heads": 4, "num_key_value_heads": 2, "intermediate_size": 172, "vocab_size": 256,
+    "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 128,
+    "tie_word_embeddings": False,
+}
+TINY_B = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 96, "num_hidden_layers": 3,
+    "num_attention_heads": 4, "num_key_value_heads": 1, "intermediate_size": 256, "vocab_size": 384,
+    "rope_theta": 500000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 256,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 32},
+    "tie_word_embeddings": True, "eos_token_id": 7,
+}
+TINY_C = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 192, "num_hidden_layers": 2,
+    "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 336,
+    "vocab_size": 500, "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 512,
+    "tie_word_embeddings": False, "rope_style": "half",
+}
+CONFIGS = {"A": (TINY_A, 0, 0.02), "B": (TINY_B, 1, 0.0), "C": (TINY_C, 2, 0.02)}
+
+_FOLDERS = {}
+_TMP = None
+
+
+def model_folder(name: str) -> str:
+    """A model folder with random bfloat16 weights for the named tiny configuration,
+    written once per test session into a temporary directory."""
+    global _TMP
+    if name not in _FOLDERS:
+        import rbitnet_amd
+        if _TMP is None:
+            _TMP = tempfile.TemporaryDirectory(prefix="rbitnet_models_")
+        cfg, seed, norm_std = CONFIGS[name]
+        folder = os.path.join(_TMP.name, name)
+        # std 0.1 rather than 0.02: with tiny widths, larger weights make attention and the
+        # gate matter, so that a wrong pairing or mask shows in the logits
+        rbitnet_amd.write_random_model(folder, cfg, seed=seed, std=0.1, norm_std=norm_std, dtype=torch.bfloat16)
+        _FOLDERS[name] = folder
+    return _FOLDERS[name]
+
+
+def tokens_for(name: str, length: int, seed: int) -> list:
+    vocab = CONFIGS[name][0]["vocab_size"]
+    rng = np.random.default_rng(1000 * seed + length)
+    return [int(t) for t in rng.integers(0, vocab, size=length)]
+
+
+@lru_cache(maxsize=None)
+def _plain(name: str):
+    from plain_llama import PlainLlama
+    return PlainLlama.from_folder(model_folder(name))
+
+
+@lru_cache(maxsize=None)
+def plain_logits(name: str, tokens: tuple) -> torch.Tensor:
+    """float64 logits [T, V] of the plain implementation (cached per sequence)."""
+    return _plain(name).logits(list(tokens))
+
+
+def max_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    """Largest absolute difference relative to the largest wanted magnitude."""
+    want = want.to(torch.float64)
+    got = got.detach().to("cpu", torch.float64)
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+# error bounds relative to the largest logit: float32 differs from the float64 oracle by
+# summation order and float32 rounding only; bfloat16 rounds activations to 8 bits of
+# mantissa at each layer boundary
+TOL = {"float32": 2e-5, "bfloat16": 3e-2}

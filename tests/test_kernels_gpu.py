@@ -1,0 +1,322 @@
+"""Each HIP kernel alone against a plain float32 (or float64) computation in torch, at
+sizes other than the engine tests use: widths that are no power of two, head sizes in
+steps of 16, odd head groups, rows that do not fill a tile."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from rbitnet_amd.csrc.lib import kernels
+    return kernels()
+
+
+def _rel(got, want):
+    want = want.double()
+    return float((got.double().cpu() - want.cpu()).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+# ------------------------------------------------------------------------ linear
+def test_reference_matvec_vectors(lib):
+    """The reference's own vectors: kernels.rs:35-40 and tests/golden_kernels.rs:12-18."""
+    w = torch.tensor([[1., 0.], [-1., 1.]], device=DEV)
+    x = torch.tensor([[2., 3.]], device=DEV)
+    c = torch.empty(1, 2, device=DEV)
+    lib.gemm_generic(x, w, c)
+    assert torch.allclose(c.cpu(), torch.tensor([[2., 1.]]), atol=1e-6)
+    w = torch.tensor([[1., -1., 0., 1.], [0., 1., 1., -1.], [1., 0., -1., 0.]], device=DEV)
+    x = torch.tensor([[0.5, -0.25, 2.0, 1.0]], device=DEV)
+    c = torch.empty(1, 3, device=DEV)
+    lib.gemm_generic(x, w, c)
+    assert torch.allclose(c.cpu(), torch.tensor([[1.75, 0.75, -1.5]]), atol=1e-5)
+    # the same through the matrix cores (K padded to 8 with zeros; values exact in bfloat16)
+    wb = torch.zeros(3, 8, device=DEV, dtype=torch.bfloat16)
+    wb[:, :4] = w.bfloat16()
+    xb = torch.zeros(1, 8, device=DEV, dtype=torch.bfloat16)
+    xb[:, :4] = x.bfloat16()
+    lib.gemm_bf16(xb, wb, c, 0)
+    assert torch.allclose(c.cpu(), torch.tensor([[1.75, 0.75, -1.5]]), atol=1e-5)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 130, 67), (65, 64, 16), (130, 200, 333)])
+def test_gemm_generic_f32(lib, m, n, k):
+    g = torch.Generator().manual_seed(m * 1000 + n)
+    a = torch.randn(m, k, generator=g)
+    w = torch.randn(n, k, generator=g)
+    c = torch.empty(m, n, device=DEV)
+    lib.gemm_generic(a.to(DEV), w.to(DEV), c)
+    assert _rel(c, a.double() @ w.double().T) < 1e-5
+
+
+@pytest.mark.parametrize("m", [1, 2, 8, 15, 16, 17, 33, 48, 64, 65, 127, 128, 200, 300])
+@pytest.mark.parametrize("n,k", [(48, 64), (100, 136), (520, 1000), (4128, 512), (20000, 72), (40000, 264)])
+def test_gemm_bf16(lib, m, n, k):
+    if m > 128 and n >= 20000:
+        pytest.skip("covered by smaller M")
+    g = torch.Generator().manual_seed(m * 7 + n)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w = torch.randn(n, k, generator=g).bfloat16()
+    want = a.double() @ w.double().T
+    for out_dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 1e-2)):
+        c = torch.full((m, n), float("nan"), device=DEV, dtype=out_dtype)
+        lib.gemm_bf16(a.to(DEV), w.to(DEV), c, 0)
+        assert _rel(c, want) < tol, (m, n, k, out_dtype)
+
+
+@pytest.mark.parametrize("m", [1, 8, 20, 64, 100, 260])
+@pytest.mark.parametrize("ff,k", [(16, 64), (336, 192), (8208, 136), (17000 // 16 * 16, 72)])
+def test_gemm_bf16_gated(lib, m, ff, k):
+    from rbitnet_amd.parts.linear import pack_gate_up
+    g = torch.Generator().manual_seed(m + ff)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    wg = (torch.randn(ff, k, generator=g) * 0.3).bfloat16()
+    wu = (torch.randn(ff, k, generator=g) * 0.3).bfloat16()
+    gate = x.double() @ wg.double().T
+    want = gate / (1 + torch.exp(-gate)) * (x.double() @ wu.double().T)
+    packed = pack_gate_up(wg, wu, True).to(DEV)
+    out = torch.full((m, ff), float("nan"), device=DEV, dtype=torch.bfloat16)
+    lib.gemm_bf16(x.to(DEV), packed, out, 1)
+    assert _rel(out, want) < 1e-2
+
+
+# ------------------------------------------------------------------------ elementwise
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed_gather(lib, dtype):
+    table = torch.randn(37, 50).to(dtype)
+    ids = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32)
+    out = torch.empty(5, 50, device=DEV)
+    lib.embed_gather(table.to(DEV), ids.to(DEV), out)
+    assert torch.equal(out.cpu(), table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("width,eps", [(50, 1e-5), (1000, 1e-6), (4100, 1e-2)])
+def test_add_rmsnorm(lib, width, eps):
+    g = torch.Generator().manual_seed(width)
+    x = torch.randn(6, width, generator=g) * 1e-2        # small, so that eps matters
+    d = torch.randn(6, width, generator=g) * 1e-2
+    w = 1 + 0.1 * torch.randn(width, generator=g)
+
+    def ref(v):
+        v = v.double()
+        return v * w.double() / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)
+
+    xd = x.to(DEV).clone()
+    out = torch.empty(6, width, device=DEV)
+    lib.add_rmsnorm(xd, None, w.to(DEV), eps, None, out)
+    assert _rel(out, ref(x)) < 1e-6
+    assert torch.equal(xd.cpu(), x)
+    lib.add_rmsnorm(xd, d.to(DEV), w.to(DEV), eps, None, out)          # adds in place
+    assert _rel(out, ref(x + d)) < 1e-6
+    assert torch.allclose(xd.cpu(), x + d, atol=0, rtol=0)
+    rows = torch.tensor([4, 1, 1], dtype=torch.int32, device=DEV)       # gather: x stays
+    xd2 = x.to(DEV).clone()
+    outb = torch.empty(3, width, device=DEV, dtype=torch.bfloat16)
+    lib.add_rmsnorm(xd2, d.to(DEV), w.to(DEV), eps, rows, outb)
+    assert torch.equal(xd2.cpu(), x)
+    assert _rel(outb, ref(x + d)[[4, 1, 1]]) < 5e-3
+    # a wrong eps, or eps outside the root, must show at this scale
+    wrong = (x + d).double() * w.double() / (torch.sqrt(((x + d).double() ** 2).mean(-1, keepdim=True)) + eps)
+    assert _rel(out, wrong) > 1e-4
+
+
+def test_swiglu(lib):
+    g = torch.Generator().manual_seed(3)
+    gu = torch.randn(5, 2 * 77, generator=g) * 4
+    out = torch.empty(5, 77, device=DEV)
+    lib.swiglu(gu.to(DEV), out)
+    gate, up = gu[:, :77].double(), gu[:, 77:].double()
+    assert _rel(out, gate / (1 + torch.exp(-gate)) * up) < 1e-6
+
+
+# ------------------------------------------------------------------------ rope + cache write, attention
+def _paged_setup(lens_past, q_lens, n_kv, d, dtype, n_pages=64, seed=0):
+    """Random q/k/v for a ragged batch and a shuffled page assignment."""
+    g = torch.Generator().manual_seed(seed)
+    b = len(q_lens)
+    total = [p + q for p, q in zip(lens_past, q_lens)]
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    tables, used = [], 0
+    for t in total:
+        n = (t + 63) // 64
+        tables.append(perm[used:used + n])
+        used += n
+    width = max(len(t) for t in tables)
+    bt = torch.tensor([t + [0] * (width - len(t)) for t in tables], dtype=torch.int32)
+    tok_seq = torch.tensor([i for i, q in enumerate(q_lens) for _ in range(q)], dtype=torch.int32)
+    tok_pos = torch.tensor([p + j for p, q in zip(lens_past, q_lens) for j in range(q)], dtype=torch.int32)
+    return g, bt, tok_seq, tok_pos, total
+
+
+def _fill_pages(k_full, v_full, bt, n_pages, n_kv, d, dtype):
+    """k_full[b]: [len, n_kv, d] -> page tensors filled with NaN where nothing is stored."""
+    kp = torch.full((n_pages, n_kv, 64, d), float("nan"), dtype=dtype)
+    vp = torch.full((n_pages, n_kv, 64, d), float("nan"), dtype=dtype)
+    for b, (kf, vf) in enumerate(zip(k_full, v_full)):
+        for p in range(kf.shape[0]):
+            page = int(bt[b, p // 64])
+            kp[page, :, p % 64] = kf[p].to(dtype)
+            vp[page, :, p % 64] = vf[p].to(dtype)
+    return kp, vp
+
+
+def _attention_ref(q, k_full, v_full, tok_seq, tok_pos, n_heads, n_kv, scale, window):
+    out = torch.zeros(q.shape[0], n_heads * q.shape[2], dtype=torch.float64)
+    d = q.shape[2]
+    for t in range(q.shape[0]):
+        b, pos = int(tok_seq[t]), int(tok_pos[t])
+        lo = 0 if not window else max(0, pos - window + 1)
+        for h in range(n_heads):
+            kvh = h // (n_heads // n_kv)
+            s = (k_full[b][lo:pos + 1, kvh].double() @ q[t, h].double()) * scale
+            p = torch.softmax(s, 0)
+            out[t, h * d:(h + 1) * d] = p @ v_full[b][lo:pos + 1, kvh].double()
+    return out
+
+
+@pytest.mark.parametrize("style", [0, 1])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_kv_write(lib, style, dtype):
+    n_heads, n_kv, d = 3, 3, 48
+    past, q_lens = [0, 70, 5], [3, 2, 60]
+    g, bt, tok_seq, tok_pos, total = _paged_setup(past, q_lens, n_kv, d, dtype)
+    t = sum(q_lens)
+    qkv = torch.randn(t, (n_heads + 2 * n_kv) * d, generator=g)
+    inv = 1.0 / (10000.0 ** (torch.arange(d // 2).double() * 2 / d))
+    ang = torch.arange(200).double()[:, None] * inv[None]
+    cos, sin = torch.cos(ang).float(), torch.sin(ang).float()
+    kp = torch.zeros(64, n_kv, 64, d, dtype=dtype, device=DEV)
+    vp = torch.zeros_like(kp)
+    qo = torch.empty(t, n_heads, d, dtype=dtype, device=DEV)
+    lib.rope_kv_write(qkv.to(DEV), cos.to(DEV), sin.to(DEV), style, qo, kp, vp, tok_pos.to(DEV), tok_seq.to(DEV),
+                      bt.to(DEV), n_heads, n_kv, d)
+    tol = 1e-6 if dtype == torch.float32 else 5e-3
+    for i in range(t):
+        pos, b = int(tok_pos[i]), int(tok_seq[i])
+        heads = qkv[i].double().view(n_heads + 2 * n_kv, d)
+        z = torch.polar(torch.ones(d // 2, dtype=torch.float64), ang[pos])          # exp(i * pos * inv)
+        if style == 0:
+            rot = torch.view_as_real(torch.view_as_complex(heads[:n_heads + n_kv].reshape(-1, d // 2, 2)) * z)
+            rot = rot.reshape(-1, d)
+        else:
+            c = torch.complex(heads[:n_heads + n_kv, :d // 2], heads[:n_heads + n_kv, d // 2:]) * z
+            rot = torch.cat([c.real, c.imag], dim=1)
+        assert _rel(qo[i], rot[:n_heads]) < tol
+        page = int(bt[b, pos // 64])
+        assert _rel(kp[page, :, pos % 64], rot[n_heads:]) < tol
+        assert _rel(vp[page, :, pos % 64], heads[n_heads + n_kv:]) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_heads,n_kv,d,window", [(3, 3, 16, 0), (6, 2, 48, 0), (4, 1, 80, 37), (5, 5, 256, 0)])
+def test_attention_generic(lib, dtype, n_heads, n_kv, d, window):
+    past, q_lens = [0, 70, 129, 63], [5, 1, 3, 66]
+    g, bt, tok_seq, tok_pos, total = _paged_setup(past, q_lens, n_kv, d, dtype, seed=d)
+    k_full = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in total]
+    v_full = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in total]
+    q = torch.randn(sum(q_lens), n_heads, d, generator=g).to(dtype)
+    kp, vp = _fill_pages(k_full, v_full, bt, 64, n_kv, d, dtype)
+    out = torch.empty(q.shape[0], n_heads * d, dtype=dtype, device=DEV)
+    scale = 1 / math.sqrt(d)
+    lib.attention_generic(q.to(DEV), kp.to(DEV), vp.to(DEV), out, tok_pos.to(DEV), tok_seq.to(DEV), bt.to(DEV),
+                          n_heads, n_kv, d, scale, window)
+    want = _attention_ref(q, k_full, v_full, tok_seq, tok_pos, n_heads, n_kv, scale, window)
+    assert _rel(out, want) < (2e-6 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("n_heads,n_kv,d,window", [(4, 1, 128, 0), (8, 8, 64, 0), (6, 3, 128, 0), (8, 1, 64, 100),
+                                                  (2, 2, 128, 70)])
+def test_attention_prefill_bf16(lib, n_heads, n_kv, d, window):
+    past, q_lens = [0, 70, 129, 0, 200], [150, 33, 3, 64, 1]
+    dtype = torch.bfloat16
+    g, bt, tok_seq, tok_pos, total = _paged_setup(past, q_lens, n_kv, d, dtype, seed=n_heads)
+    k_full = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in total]
+    v_full = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in total]
+    q = (torch.randn(sum(q_lens), n_heads, d, generator=g) * 2).to(dtype)
+    kp, vp = _fill_pages(k_full, v_full, bt, 64, n_kv, d, dtype)
+    out = torch.full((q.shape[0], n_heads * d), float("nan"), dtype=dtype, device=DEV)
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    scale = 1 / math.sqrt(d)
+    lib.attention_prefill_bf16(q.to(DEV), kp.to(DEV), vp.to(DEV), out, cu.to(DEV),
+                               torch.tensor(past, dtype=torch.int32, device=DEV), bt.to(DEV), len(q_lens),
+                               max(q_lens), n_heads, n_kv, d, scale, window)
+    want = _attention_ref(q, k_full, v_full, tok_seq, tok_pos, n_heads, n_kv, scale, window)
+    assert _rel(out, want) < 1.5e-2
+
+
+@pytest.mark.parametrize("n_heads,n_kv,d,window,n_splits", [(4, 1, 128, 0, 3), (8, 8, 64, 0, 1), (8, 4, 128, 0, 8),
+                                                           (8, 1, 64, 90, 2), (2, 2, 128, 65, 5)])
+def test_attention_decode_bf16(lib, n_heads, n_kv, d, window, n_splits):
+    past, q_lens = [0, 70, 129, 63, 64, 300], [1, 1, 1, 1, 1, 1]
+    dtype = torch.bfloat16
+    g, bt, tok_seq, tok_pos, total = _paged_setup(past, q_lens, n_kv, d, dtype, seed=n_heads + 1)
+    k_full = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in total]
+    v_full = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in total]
+    q = (torch.randn(len(q_lens), n_heads, d, generator=g) * 2).to(dtype)
+    kp, vp = _fill_pages(k_full, v_full, bt, 64, n_kv, d, dtype)
+    out = torch.full((q.shape[0], n_heads * d), float("nan"), dtype=dtype, device=DEV)
+    ws = torch.full((len(q_lens) * n_heads * n_splits * (d + 2),), float("nan"), device=DEV)
+    scale = 1 / math.sqrt(d)
+    lib.attention_decode_bf16(q.to(DEV), kp.to(DEV), vp.to(DEV), out, tok_pos.to(DEV), bt.to(DEV), n_heads, n_kv, d,
+                              scale, window, n_splits, ws)
+    want = _attention_ref(q, k_full, v_full, tok_seq, tok_pos, n_heads, n_kv, scale, window)
+    assert _rel(out, want) < 1e-2
+
+
+def test_far_key_stands_out(lib):
+    """One key among hundreds, scaled so that its score dominates: the output must be that
+    key's value, wherever it lies (first page, page edge, last position)."""
+    n_heads, n_kv, d = 4, 1, 128
+    dtype = torch.bfloat16
+    total = 700
+    for target in (0, 63, 64, 511, 698, 699):
+        g, bt, tok_seq, tok_pos, _ = _paged_setup([total - 1], [1], n_kv, d, dtype, seed=target)
+        k = torch.randn(total, n_kv, d, generator=g) * 0.1
+        v = torch.randn(total, n_kv, d, generator=g)
+        q = torch.randn(1, n_heads, d, generator=g) * 0.1
+        k[target, 0] = 40 * q[0, 1] / q[0, 1].norm()          # head 1 looks at `target`
+        q[0, 1] = 40 * q[0, 1] / q[0, 1].norm()
+        kp, vp = _fill_pages([k], [v], bt, 64, n_kv, d, dtype)
+        scale = 1 / math.sqrt(d)
+        outs = []
+        out = torch.empty(1, n_heads * d, dtype=dtype, device=DEV)
+        lib.attention_generic(q.to(dtype).to(DEV), kp.to(DEV), vp.to(DEV), out, tok_pos.to(DEV), tok_seq.to(DEV),
+                              bt.to(DEV), n_heads, n_kv, d, scale, 0)
+        outs.append(out.clone())
+        ws = torch.empty(n_heads * 4 * (d + 2), device=DEV)
+        lib.attention_decode_bf16(q.to(dtype).to(DEV), kp.to(DEV), vp.to(DEV), out, tok_pos.to(DEV), bt.to(DEV),
+                                  n_heads, n_kv, d, scale, 0, 4, ws)
+        outs.append(out.clone())
+        cu = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
+        lib.attention_prefill_bf16(q.to(dtype).to(DEV), kp.to(DEV), vp.to(DEV), out, cu,
+                                   torch.tensor([total - 1], dtype=torch.int32, device=DEV), bt.to(DEV), 1, 1,
+                                   n_heads, n_kv, d, scale, 0)
+        outs.append(out.clone())
+        for o in outs:
+            got = o[0, d:2 * d].float().cpu()
+            assert (got - v[target, 0].to(dtype).float()).abs().max() < 2e-2, target
+
+
+# ------------------------------------------------------------------------ sampling
+def test_sample_greedy_and_inverse_cdf(lib):
+    from plain_llama import sample_token
+    g = torch.Generator().manual_seed(11)
+    logits = torch.randn(7, 1000, generator=g) * 3
+    logits[2, 5] = logits[2, 900] = 50.0                 # equal maxima: the lowest index wins
+    logits[3, 17] = float("nan")
+    tokens = torch.empty(7, dtype=torch.int32, device=DEV)
+    lib.sample(logits.to(DEV), None, None, tokens)
+    want = [int(torch.nan_to_num(r, nan=-float("inf")).argmax()) for r in logits]
+    want[2] = 5
+    assert tokens.tolist() == want
+    temps = torch.tensor([0.8, 0.0, 1.5, 0.3, 1.0, 0.8, 2.0])
+    us = torch.tensor([0.0, 0.5, 0.999999, 0.25, 0.5, 0.73, 0.1])
+    lib.sample(logits.to(DEV), temps.to(DEV), us.to(DEV), tokens)
+    for r in range(7):
+        row = torch.nan_to_num(logits[r], nan=-float("inf"))
+        assert tokens[r].item() == sample_token(row, float(temps[r]), float(us[r])), r
