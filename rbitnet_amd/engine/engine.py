@@ -159,6 +159,12 @@ class Engine:
             self.stats["prefill_tokens"] += sum(q_lens)
         return logits
 
+    def decode_step(self, slots: Sequence[int], tokens: Sequence[int], temperatures=None, uniforms=None) -> list:
+        """One token per sequence in, the next token per sequence out: a step and the
+        sampling of its logits."""
+        logits = self.step([(s, [t]) for s, t in zip(slots, tokens)], "last")
+        return self.sampler.sample(logits, temperatures, uniforms)
+
     # ------------------------------------------------------------------ generation
     def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 256, temperature: float = 0.7,
                  seed: int = 0, stop_token_ids: Optional[Sequence[int]] = None):
