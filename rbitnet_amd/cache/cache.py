@@ -64,8 +64,9 @@ class StateGroup:
 class Cache:
     def __init__(self, requests: Sequence[Optional[CacheRequest]], n_slots: int, max_tokens: int,
                  dtype: torch.dtype, device, readers: Optional[Dict[int, int]] = None):
-        """requests[l]: what layer l's mixer asked for (None: nothing).  readers[l] = j:
-        layer l reads layer j's keys and values.  max_tokens: positions the pages of each
+        """requests[l]: what the mixer at place l of the schedule asked for (None: nothing);
+        "layer" below means such a place.  readers[l] = j: place l reads place j's keys and
+        values.  max_tokens: positions the pages of each
         group hold together, every sequence rounded up to whole pages."""
         if n_slots <= 0:
             raise CacheError("the cache needs at least one slot")

@@ -69,6 +69,16 @@ class Engine:
         return cls(cfg, spec, model, max_tokens=max_tokens, max_batch=max_batch, max_seq_len=seq)
 
     @classmethod
+    def from_spec(cls, spec, tensors, dtype: Any = "bfloat16", max_tokens: int = 4096, max_batch: int = 8,
+                  max_seq_len: Optional[int] = None, device: str = "cuda:0", generic_only: bool = False) -> "Engine":
+        """An engine from a hand-made `ModelSpec` and tensors by name: what a new
+        architecture's configuration class would produce, without one."""
+        from ..csrc.lib import kernels
+        model = Model(spec, parse_dtype(dtype), device, kernels(), generic_only=generic_only)
+        model.load(tensors)
+        return cls(None, spec, model, max_tokens=max_tokens, max_batch=max_batch, max_seq_len=max_seq_len)
+
+    @classmethod
     def load_path(cls, path: str, dtype: Any = "bfloat16", max_tokens: Optional[int] = None,
                   max_batch: Optional[int] = None, max_seq_len: Optional[int] = None, device: str = "cuda:0",
                   generic_only: bool = False) -> "Engine":

@@ -84,18 +84,32 @@ class Model:
 
     # ------------------------------------------------------------------ cache needs
     def cache_requests(self) -> List[Optional[CacheRequest]]:
+        """One entry per place in the schedule: a layer that runs twice keeps two caches,
+        since its second run sees other inputs than its first."""
         out = []
-        for b in self.blocks:
-            req = getattr(b.mixer, "cache_request", None)
+        for i in self.spec.schedule:
+            req = getattr(self.blocks[i].mixer, "cache_request", None)
             out.append(req() if req else None)
         return out
 
     def cache_readers(self) -> Dict[int, int]:
+        """place in the schedule -> the place whose keys and values it reads: the latest
+        earlier run of the layer that its mixer's `cache_from` names."""
         out = {}
-        for i, b in enumerate(self.blocks):
-            j = getattr(b.mixer, "cache_from", None)
-            if j is not None:
-                out[i] = int(j)
+        for place, i in enumerate(self.spec.schedule):
+            j = getattr(self.blocks[i].mixer, "cache_from", None)
+            if j is None:
+                continue
+            earlier = [p for p in range(place) if self.spec.schedule[p] == int(j)]
+            if not earlier:
+                raise ConfigError(f"layer {i} reads the cache of layer {j}, which does not run before it")
+            out[place] = earlier[-1]
+            own = getattr(self.blocks[i].mixer, "window", None)
+            theirs = getattr(self.blocks[int(j)].mixer, "window", None)
+            if theirs is not None and (own is None or int(own) > int(theirs)):
+                raise ConfigError(
+                    f"layer {i} looks back {own or 'without limit'} but reads the cache of layer {j}, "
+                    f"which keeps only the last {theirs} positions")
         return out
 
     def max_positions(self) -> int:
@@ -146,7 +160,7 @@ class Model:
         x = torch.empty((ctx.n_tokens, self.spec.hidden_size), dtype=torch.float32, device=self.device)
         self.lib.embed_gather(self.embedding, ctx.token_ids, x)
         pending = None
-        for i in self.spec.schedule:
-            pending = self.blocks[i].forward(x, pending, ctx, cache.view(i, ctx.block_tables))
+        for place, i in enumerate(self.spec.schedule):
+            pending = self.blocks[i].forward(x, pending, ctx, cache.view(place, ctx.block_tables))
         xn = self.final_norm.forward(x, pending, rows)
         return linear(self.lib, xn, self.head, torch.float32)

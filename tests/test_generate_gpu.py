@@ -1,0 +1,169 @@
+"""Generation through the Python entry point and the command line, long decoding, the
+first tokens of a sequence, sampling that does not depend on the batch."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from helpers import TOL, max_err, model_folder, plain_logits, tokens_for
+from plain_llama import argmax_token, sample_token
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _engine(name, dtype, **kw):
+    import rbitnet_amd
+    kw.setdefault("max_tokens", 2048)
+    return rbitnet_amd.Engine.load_path(model_folder(name), dtype=dtype, **kw)
+
+
+def _plain_greedy(name, prompt, n, stop=()):
+    """Greedy continuation by the plain implementation, with the margin between the best
+    and the second logit at each step (a tiny margin means either token is right)."""
+    seq, out, margins = list(prompt), [], []
+    for _ in range(n):
+        row = plain_logits(name, tuple(seq))[-1]
+        top = torch.topk(row, 2).values
+        tok = argmax_token(row)
+        if tok in stop:
+            break
+        margins.append(float(top[0] - top[1]))
+        out.append(tok)
+        seq.append(tok)
+    return out, margins
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_matches_plain_float32(name):
+    eng = _engine(name, "float32", max_batch=3)
+    prompts = [tokens_for(name, n, 40 + i) for i, n in enumerate([5, 17, 32, 1])]
+    results = eng.generate(prompts, max_tokens=16, temperature=0.0, stop_token_ids=[])
+    for p, r in zip(prompts, results):
+        want, margins = _plain_greedy(name, p, 16)
+        assert min(margins) > 1e-4, "test data: a near tie, pick another seed"
+        assert r.tokens == want and r.finish_reason == "length"
+    # the same call twice gives the same tokens (the reference's determinism test, toy.rs:121-127)
+    again = eng.generate(prompts, max_tokens=16, temperature=0.0, stop_token_ids=[])
+    assert [r.tokens for r in again] == [r.tokens for r in results]
+    assert eng.cache.slots.n_held == 0
+    eng.cache.check()
+
+
+def test_stop_token_ends_generation_and_is_not_emitted():
+    eng = _engine("A", "float32")
+    prompt = tokens_for("A", 9, 3)
+    want, _ = _plain_greedy("A", prompt, 12)
+    stop = want[4]
+    first = want.index(stop)
+    (r,) = eng.generate([prompt], max_tokens=12, temperature=0.0, stop_token_ids=[stop])
+    assert r.tokens == want[:first] and r.finish_reason == "stop"
+
+
+def test_bfloat16_greedy_agrees_where_the_margin_is_clear():
+    eng = _engine("C", "bfloat16")
+    prompt = tokens_for("C", 20, 5)
+    (r,) = eng.generate([prompt], max_tokens=24, temperature=0.0, stop_token_ids=[])
+    seq = list(prompt)
+    for tok in r.tokens:                       # follow the engine's own path and judge each choice
+        row = plain_logits("C", tuple(seq))[-1]
+        best = argmax_token(row)
+        if tok != best:
+            assert float(row[best] - row[tok]) < 0.05 * float(row.abs().max()), "a clear best token was missed"
+        seq.append(tok)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(dtype):
+    """A short prompt and then 300 tokens one by one across several pages: every logit row
+    against the plain implementation run on the whole sequence."""
+    name = "C"
+    toks = tokens_for(name, 310, 77)
+    want = plain_logits(name, tuple(toks))
+    eng = _engine(name, dtype)
+    slot = eng.alloc_slot()
+    rows = [eng.step([(slot, toks[:10])], "all")]
+    for t in toks[10:]:
+        rows.append(eng.step([(slot, [t])], "last"))
+    eng.free_slot(slot)
+    got = torch.cat(rows).cpu().double()
+    err = (got - want).abs().amax(dim=1) / want.abs().max()
+    assert float(err.max()) < TOL[dtype], f"worst position {int(err.argmax())}: {float(err.max())}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens_of_a_sequence(name, dtype):
+    """Positions 0, 1, 2 alone and together: a one-token sequence attends to itself only."""
+    toks = tokens_for(name, 3, 9)
+    want = plain_logits(name, tuple(toks))
+    eng = _engine(name, dtype)
+    for cut in ([3], [1, 2], [1, 1, 1], [2, 1]):
+        slot = eng.alloc_slot()
+        rows, at = [], 0
+        for n in cut:
+            rows.append(eng.step([(slot, toks[at:at + n])], "all"))
+            at += n
+        eng.free_slot(slot)
+        assert max_err(torch.cat(rows), want) < TOL[dtype], cut
+
+
+def test_temperature_sampling_does_not_depend_on_the_batch():
+    eng = _engine("B", "float32", max_batch=4)
+    prompts = [tokens_for("B", n, 60 + i) for i, n in enumerate([1, 9, 40, 77])]
+    together = eng.generate(prompts, max_tokens=24, temperature=0.8, seed=5, stop_token_ids=[])
+    eng1 = _engine("B", "float32", max_batch=1)
+    alone = eng1.generate(prompts, max_tokens=24, temperature=0.8, seed=5, stop_token_ids=[])
+    assert [r.tokens for r in together] == [r.tokens for r in alone]
+    other = eng.generate(prompts, max_tokens=24, temperature=0.8, seed=6, stop_token_ids=[])
+    assert [r.tokens for r in other] != [r.tokens for r in together]
+    # the first sampled token of each request against the plain inverse CDF
+    from rbitnet_amd.sampling import uniform
+    for i, (p, r) in enumerate(zip(prompts, together)):
+        row = plain_logits("B", tuple(p))[-1]
+        assert r.tokens[0] == sample_token(row, 0.8, uniform(5, i, 0))
+
+
+def test_step_refuses_what_it_cannot_run():
+    from rbitnet_amd.errors import CacheError, InferenceError
+    eng = _engine("A", "float32", max_tokens=128, max_batch=2)
+    s = eng.alloc_slot()
+    with pytest.raises(InferenceError, match="token id out of range"):
+        eng.step([(s, [256])])
+    with pytest.raises(InferenceError, match="position >= max_seq"):
+        eng.step([(s, [1] * 129)])
+    with pytest.raises(InferenceError, match="at least one token"):
+        eng.step([(s, [])])
+    with pytest.raises(InferenceError, match="wanted place"):
+        eng.step([(s, [1, 2])], [[2]])
+    assert eng.length(s) == 0
+    s2 = eng.alloc_slot()
+    eng.step([(s, [1] * 70)])
+    with pytest.raises(CacheError, match="cache full"):
+        eng.step([(s2, [1])])                  # both pages are held by the first sequence
+    with pytest.raises(CacheError):
+        eng.alloc_slot()
+    eng.free_slot(s)
+    eng.step([(s2, [1])])
+
+
+def test_command_line_generate_and_inspect(tmp_path):
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    folder = model_folder("A")
+    prompt = tokens_for("A", 7, 21)
+    want, _ = _plain_greedy("A", prompt, 5)
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "rbitnet"), "generate", "--model", folder,
+                          "--dtype", "float32", "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "5",
+                          "--temperature", "0"], capture_output=True, text=True, env=env, timeout=300)
+    assert out.returncode == 0, out.stderr
+    rec = json.loads(out.stdout.strip().splitlines()[-1])
+    assert rec["tokens"] == want and rec["finish_reason"] == "length" and rec["prompt_tokens"] == 7
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "rbitnet"), "generate", "--model",
+                          str(tmp_path / "none"), "--prompt-ids", "1"], capture_output=True, text=True, env=env)
+    assert bad.returncode == 1 and bad.stderr.startswith("error: ")
+    ins = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "rbitnet"), "inspect", folder],
+                         capture_output=True, text=True, env=env)
+    assert ins.returncode == 0 and "tensors=21" in ins.stdout and "... and 1 more" in ins.stdout

@@ -1,0 +1,262 @@
+"""Each part alone against the plain functions, and the generality of the composition:
+a toy mixer with state of its own, defined here, registered, built and stepped without a
+change to the framework; layers of different kinds and sizes in one model; a layer that
+runs twice; a layer that reads another layer's cache; a window."""
+import math
+
+import pytest
+import torch
+
+import plain_llama as P
+from rbitnet_amd.cache import Cache
+from rbitnet_amd.config.spec import LayerSpec, ModelSpec, PartSpec
+from rbitnet_amd.engine.context import StepContext
+from rbitnet_amd.parts import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register_mixer
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+D64 = torch.float64
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from rbitnet_amd.csrc.lib import kernels
+    return kernels()
+
+
+def _env(lib, hidden, dtype):
+    return BuildEnv(hidden_size=hidden, dtype=dtype, device=torch.device(DEV), lib=lib)
+
+
+def _rel(got, want):
+    want = want.double().cpu()
+    return float((got.double().cpu() - want).abs().max() / want.abs().max())
+
+
+def _ctx_and_cache(part, past, tokens_per_seq, dtype):
+    """A cache for one mixer and a step context for sequences with `past` tokens already
+    stored (the caller fills them by running earlier steps)."""
+    cache = Cache([part.cache_request()], len(past), 64 * 16, dtype, DEV)
+    slots = [cache.alloc_slot() for _ in past]
+    return cache, slots
+
+
+def _step(cache, slots, q_lens):
+    past = [cache.length(s) for s in slots]
+    cache.reserve(slots, q_lens)
+    tables = {id(g): cache.block_table(g, slots) for g in cache.kv_groups}
+    ctx = StepContext(DEV, slots, past, [[0] * q for q in q_lens], [], tables)
+    return ctx
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-6), (torch.bfloat16, 8e-3)])
+def test_norm_part(lib, dtype, tol):
+    part = build_part("norm", PartSpec("rmsnorm", {"size": 100, "eps": 1e-3}), _env(lib, 100, dtype))
+    assert part.tensor_specs()["weight"].shape == (100,) and part.tensor_specs()["weight"].role == "gain"
+    w = 1 + 0.2 * torch.randn(100)
+    part.load({"weight": w.to(DEV)})
+    x, d = torch.randn(5, 100) * 0.03, torch.randn(5, 100) * 0.03
+    xd = x.to(DEV).clone()
+    got = part.forward(xd, d.to(DEV))
+    assert got.dtype == dtype and _rel(got, P.rmsnorm((x + d).double(), w.double(), 1e-3)) < tol
+    assert torch.equal(xd.cpu(), x + d)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 2e-2)])
+def test_feed_forward_part(lib, dtype, tol):
+    for hidden, ff in ((40, 52), (64, 96)):              # generic path, then the fused matrix-core path
+        part = build_part("feed_forward", PartSpec("swiglu", {"intermediate_size": ff}), _env(lib, hidden, dtype))
+        names = part.names
+        w = {names["gate"]: torch.randn(ff, hidden) * 0.3, names["up"]: torch.randn(ff, hidden) * 0.3,
+             names["down"]: torch.randn(hidden, ff) * 0.3}
+        w = {k: v.to(dtype) for k, v in w.items()}
+        part.load({k: v.to(DEV) for k, v in w.items()})
+        h = torch.randn(7, hidden).to(dtype)
+        got = part.forward(h.to(DEV))
+        want = P.swiglu(h.double(), w[names["gate"]].double(), w[names["up"]].double(), w[names["down"]].double())
+        assert got.dtype == torch.float32 and _rel(got, want) < tol, (hidden, ff)
+
+
+def _attention_params(hq, hk, d, window=None, theta=10000.0, style="interleaved", scaling=None):
+    return {"num_heads": hq, "num_kv_heads": hk, "head_dim": d, "scale": 1 / math.sqrt(d), "window": window,
+            "cache_from": None,
+            "position": PartSpec("rope", {"head_dim": d, "theta": theta, "scaling": scaling, "style": style,
+                                          "max_positions": 512})}
+
+
+def _plain_attention_layer(h, w, names, hq, hk, d, theta, style, window):
+    q, k, v = (P.linear(h, w[names[n]].double()) for n in ("q", "k", "v"))
+    inv = P.rope_inv_freq(d, theta, None)
+    for pos in range(h.shape[0]):
+        for i in range(hq):
+            q[pos, i * d:(i + 1) * d] = P.rope(q[pos, i * d:(i + 1) * d], pos, inv, style)
+        for i in range(hk):
+            k[pos, i * d:(i + 1) * d] = P.rope(k[pos, i * d:(i + 1) * d], pos, inv, style)
+    return P.linear(P.attention(q, k, v, hq, hk, window), w[names["o"]].double())
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-6), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("hq,hk,d,window,style", [(6, 3, 10, None, "interleaved"), (4, 1, 64, None, "half"),
+                                                  (8, 2, 128, 50, "interleaved"), (2, 2, 32, 7, "half")])
+def test_attention_part_whole_and_in_pieces(lib, dtype, tol, hq, hk, d, window, style):
+    hidden = 48
+    part = build_part("mixer", PartSpec("attention", _attention_params(hq, hk, d, window, style=style)),
+                      _env(lib, hidden, dtype))
+    specs = part.tensor_specs()
+    w = {n: (torch.randn(s.shape) * 0.2).to(dtype) for n, s in specs.items()}
+    part.load({n: t.to(DEV) for n, t in w.items()})
+    t_len = 150
+    h = torch.randn(t_len, hidden).to(dtype)
+    want = _plain_attention_layer(h.double(), w, part.names, hq, hk, d, 10000.0, style, window)
+    for cuts in ([t_len], [100, 1, 1, 48], [64, 64, 22]):
+        cache, slots = _ctx_and_cache(part, [0], None, dtype)
+        outs, at = [], 0
+        for n in cuts:
+            ctx = _step(cache, slots, [n])
+            view = cache.view(0, ctx.block_tables)
+            outs.append(part.forward(h[at:at + n].to(DEV).contiguous(), ctx, view))
+            cache.commit(slots, [n])
+            at += n
+        assert _rel(torch.cat(outs), want) < tol, cuts
+
+
+# ---------------------------------------------------------------------------- a toy mixer with state
+class DecayMixer(Part):
+    """s_t = a * s_{t-1} + h_t per sequence (a fixed-size state, no keys or values),
+    out_t = W s_t.  Written with torch operations: the framework only has to hand it its
+    state and the batch's layout."""
+
+    def __init__(self, params, env):
+        self.env, self.a, self.hidden = env, float(params["decay"]), env.hidden_size
+
+    def tensor_specs(self):
+        return {"mix.weight": TensorSpec((self.hidden, self.hidden))}
+
+    def load(self, tensors):
+        self.w = tensors["mix.weight"]
+
+    def cache_request(self):
+        return CacheRequest("state", state_shape=(self.hidden,), state_init=0.0)
+
+    def forward(self, h, ctx, view):
+        hf = h.float()
+        out = torch.empty_like(hf)
+        cu = ctx.cu_seqlens.tolist()
+        for b, slot in enumerate(ctx.host_slots):
+            s = view.state[slot]
+            for t in range(cu[b], cu[b + 1]):
+                s = self.a * s + hf[t]
+                out[t] = s
+            view.state[slot] = s
+        return out @ self.w.float().T
+
+
+def _plain_toy_model(spec, tensors, tokens):
+    """The hand-made model of test_toy_mixer... computed plainly in float64."""
+    w = {k: v.double().cpu() for k, v in tensors.items()}
+    x = P.embedding(w[spec.embedding_name], tokens)
+    states = {}
+    for place, i in enumerate(spec.schedule):
+        layer = spec.layers[i]
+        pre = layer.prefix
+        h = P.rmsnorm(x, w[f"{pre}.input_layernorm.weight"], layer.norm1["eps"])
+        if layer.mixer.kind == "toy_decay":
+            s = torch.zeros(spec.hidden_size, dtype=D64)
+            rows = []
+            for t in range(h.shape[0]):
+                s = layer.mixer["decay"] * s + h[t]
+                rows.append(s)
+            a = P.linear(torch.stack(rows), w[f"{pre}.self_attn.mix.weight"])
+            states[place] = None
+        else:
+            m = layer.mixer
+            hq, hk, d = m["num_heads"], m["num_kv_heads"], m["head_dim"]
+            inv = P.rope_inv_freq(d, m["position"]["theta"], None)
+            q = P.linear(h, w[f"{pre}.self_attn.q_proj.weight"])
+            for pos in range(h.shape[0]):
+                for j in range(hq):
+                    q[pos, j * d:(j + 1) * d] = P.rope(q[pos, j * d:(j + 1) * d], pos, inv)
+            if m["cache_from"] is None:
+                k = P.linear(h, w[f"{pre}.self_attn.k_proj.weight"])
+                v = P.linear(h, w[f"{pre}.self_attn.v_proj.weight"])
+                for pos in range(h.shape[0]):
+                    for j in range(hk):
+                        k[pos, j * d:(j + 1) * d] = P.rope(k[pos, j * d:(j + 1) * d], pos, inv)
+                states[place] = (k, v)
+            else:
+                src = [p for p in range(place) if spec.schedule[p] == m["cache_from"]][-1]
+                k, v = states[src]
+            a = P.linear(P.attention(q, k, v, hq, hk, m["window"]), w[f"{pre}.self_attn.o_proj.weight"])
+        x = x + a
+        h2 = P.rmsnorm(x, w[f"{pre}.post_attention_layernorm.weight"], layer.norm2["eps"])
+        x = x + P.swiglu(h2, w[f"{pre}.mlp.gate_proj.weight"], w[f"{pre}.mlp.up_proj.weight"],
+                         w[f"{pre}.mlp.down_proj.weight"])
+    xn = P.rmsnorm(x, w[spec.final_norm_name], spec.final_norm["eps"])
+    return P.linear(xn, w[spec.head_name])
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_toy_mixer_and_mixed_layers(dtype, tol):
+    """Layer 0: windowed attention.  Layer 1: the toy state mixer with a wider
+    feed-forward.  Layer 2: attention that reads layer 0's cache, other eps.  Schedule
+    0, 1, 2, 1: layer 1 runs twice, with a state per run."""
+    import rbitnet_amd
+    from rbitnet_amd.engine.model import expected_tensors
+    from rbitnet_amd.weights import random_tensors
+    register_mixer("toy_decay", DecayMixer)
+    hidden, vocab = 48, 90
+    norm = lambda eps: PartSpec("rmsnorm", {"size": hidden, "eps": eps})
+    att0 = _attention_params(4, 2, 16, window=40)
+    att2 = dict(_attention_params(4, 2, 16, window=33), cache_from=0)
+    layers = [
+        LayerSpec("blocks.0", "prenorm", PartSpec("attention", att0), PartSpec("swiglu", {"intermediate_size": 64}),
+                  norm(1e-5), norm(1e-5)),
+        LayerSpec("blocks.1", "prenorm", PartSpec("toy_decay", {"decay": 0.7}),
+                  PartSpec("swiglu", {"intermediate_size": 100}), norm(1e-5), norm(1e-5)),
+        LayerSpec("blocks.2", "prenorm", PartSpec("attention", att2), PartSpec("swiglu", {"intermediate_size": 32}),
+                  norm(1e-3), norm(1e-3)),
+    ]
+    spec = ModelSpec(architecture="ToyForTests", hidden_size=hidden, vocab_size=vocab, max_positions=512,
+                     embedding_name="embed.weight", layers=layers, final_norm=norm(1e-5),
+                     final_norm_name="final_norm.weight", head_name="head.weight", schedule=[0, 1, 2, 1])
+    # a reader must not look further back than the cache it reads keeps
+    bad = ModelSpec(architecture="ToyForTests", hidden_size=hidden, vocab_size=vocab, max_positions=512,
+                    embedding_name="embed.weight", final_norm=norm(1e-5), final_norm_name="final_norm.weight",
+                    head_name="head.weight", layers=[layers[0], LayerSpec(
+                        "blocks.1", "prenorm", PartSpec("attention", dict(att2, window=None)),
+                        PartSpec("swiglu", {"intermediate_size": 32}), norm(1e-5), norm(1e-5))])
+    from rbitnet_amd.engine.model import Model
+    from rbitnet_amd.errors import ConfigError
+    with pytest.raises(ConfigError, match="keeps only the last 40"):
+        Model(bad, torch.float32, DEV, None).cache_readers()
+    expected = expected_tensors(spec)
+    assert "blocks.1.self_attn.mix.weight" in expected and "blocks.2.self_attn.k_proj.weight" not in expected
+    tensors = dict(random_tensors(expected, seed=4, std=0.15, norm_std=0.05, dtype=torch.bfloat16))
+    eng = rbitnet_amd.Engine.from_spec(spec, tensors, dtype=dtype, max_tokens=64 * 12, max_batch=3)
+    assert len(eng.cache.kv_groups) == 1 and len(eng.cache.state_groups) == 1
+    assert eng.cache.state_groups[0].data.shape[0] == 2            # two runs of layer 1, two states
+    g = torch.Generator().manual_seed(8)
+    seqs = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in (130, 9, 70)]
+    want = [_plain_toy_model(spec, tensors, s) for s in seqs]
+    # whole
+    for s, w in zip(seqs, want):
+        slot = eng.alloc_slot()
+        assert _rel(eng.step([(slot, s)], "all"), w) < tol
+        eng.free_slot(slot)
+    # as a batch: unequal prompts, then one token each; slots used again (state must be reset)
+    slots = [eng.alloc_slot() for _ in seqs]
+    cut = [len(s) - 5 for s in seqs]
+    logits = eng.step([(sl, s[:c]) for sl, s, c in zip(slots, seqs, cut)], "all")
+    off = 0
+    for s, c, w in zip(seqs, cut, want):
+        assert _rel(logits[off:off + c], w[:c]) < tol
+        off += c
+    for j in range(5):
+        logits = eng.step([(sl, [s[c + j]]) for sl, s, c in zip(slots, seqs, cut)], "last")
+        for i, (c, w) in enumerate(zip(cut, want)):
+            assert _rel(logits[i:i + 1], w[c + j:c + j + 1]) < tol * 2
+    for sl in slots:
+        eng.free_slot(sl)
+    eng.cache.check()
+    # the windowed group gave pages back while the long sequence ran
+    assert eng.cache.kv_groups[0].table.pool.n_free == eng.cache.n_pages
