@@ -19,7 +19,7 @@
 #include "mfma.h"
 
 // =============================================================================== skinny
-template <int MB, int R, int EPI, typename TO>
+template <int MB, int R, int U, bool FAST, int EPI, typename TO>
 __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                           const bf16_t* __restrict__ w, TO* __restrict__ c,
                                                           int m, int n, int k, int k_per_wave) {
@@ -57,23 +57,64 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
 
   const int k_begin = wave * k_per_wave;
   const int k_end = (k_begin + k_per_wave < k) ? k_begin + k_per_wave : k;
-  for (int k0 = k_begin; k0 < k_end; k0 += 128) {
-    Frag8 a[R][4], b[MB][4];
+  if (FAST) {
+    // K and every wave's range are multiples of 128: no bounds checks.  Rows beyond N or M
+    // are read from row 0 instead and their results never stored.  U stages of 128 depth
+    // values stay in flight: as soon as a stage has been multiplied, its registers are
+    // loaded again with the stage U further on.
+    // The host chose the waves so that every wave has the same number of stages, a
+    // positive multiple of U: the loads below are unconditional, which lets the compiler
+    // count outstanding loads exactly and start multiplying when the oldest stage arrives.
+    const int stages = k_per_wave / 128;
+    Frag8 a[U][R][4], b[U][MB][4];
+    auto load_stage = [&](int u, int st) {
+      const int kk = k_begin + 128 * st + 8 * kq;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int kk = k0 + 32 * j + 8 * kq;
-      const bool in = kk < k_end;
+      for (int j = 0; j < 4; ++j) {
 #pragma unroll
-      for (int rt = 0; rt < R; ++rt) a[rt][j].u = (in && wok[rt]) ? load16(wrow[rt] + kk) : zero16();
+        for (int rt = 0; rt < R; ++rt) a[u][rt][j].u = load16(wrow[rt] + kk + 32 * j);
 #pragma unroll
-      for (int cb = 0; cb < MB; ++cb) b[cb][j].u = (in && xok[cb]) ? load16(xrow[cb] + kk) : zero16();
+        for (int cb = 0; cb < MB; ++cb) b[u][cb][j].u = load16(xrow[cb] + kk + 32 * j);
+      }
+    };
+    auto multiply_stage = [&](int u) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+          for (int cb = 0; cb < MB; ++cb) acc[rt][cb] = mfma16(a[u][rt][j], b[u][cb][j], acc[rt][cb]);
+    };
+#pragma unroll
+    for (int u = 0; u < U; ++u) load_stage(u, u);
+    for (int s0 = 0; s0 + U < stages; s0 += U) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        multiply_stage(u);
+        load_stage(u, s0 + u + U);
+      }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int u = 0; u < U; ++u) multiply_stage(u);
+  } else {
+    for (int k0 = k_begin; k0 < k_end; k0 += 128) {
+      Frag8 a[R][4], b[MB][4];
 #pragma unroll
-      for (int rt = 0; rt < R; ++rt)
+      for (int j = 0; j < 4; ++j) {
+        const int kk = k0 + 32 * j + 8 * kq;
+        const bool in = kk < k_end;
 #pragma unroll
-        for (int cb = 0; cb < MB; ++cb) acc[rt][cb] = mfma16(a[rt][j], b[cb][j], acc[rt][cb]);
+        for (int rt = 0; rt < R; ++rt) a[rt][j].u = (in && wok[rt]) ? load16(wrow[rt] + kk) : zero16();
+#pragma unroll
+        for (int cb = 0; cb < MB; ++cb) b[cb][j].u = (in && xok[cb]) ? load16(xrow[cb] + kk) : zero16();
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+          for (int cb = 0; cb < MB; ++cb) acc[rt][cb] = mfma16(a[rt][j], b[cb][j], acc[rt][cb]);
+    }
   }
 
   // ---- partial sums of waves 1.. go through LDS to wave 0
@@ -133,18 +174,52 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
   }
 }
 
-template <int MB, int R, int EPI, typename TO>
-static int launch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
-  int n_waves = k / 256;
-  if (n_waves < 1) n_waves = 1;
-  if (n_waves > 8) n_waves = 8;
-  int k_per_wave = (k + n_waves - 1) / n_waves;
-  k_per_wave = (k_per_wave + 127) / 128 * 128;
+static int g_tune_u = 0, g_tune_r = 0, g_tune_waves = 0;
+extern "C" void rb_tune(int u, int r, int waves) {       // experiments only; 0 = the built-in choice
+  g_tune_u = u;
+  g_tune_r = r;
+  g_tune_waves = waves;
+}
+
+template <int MB, int R, int U, bool FAST, int EPI, typename TO>
+static int launch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, int n_waves,
+                         int k_per_wave, hipStream_t s) {
   const size_t lds = (size_t)(n_waves - 1) * R * MB * 4 * 64 * sizeof(float);
   RB_REQUIRE(lds <= 64 * 1024, "rb_gemm_bf16: internal: reduction buffer of %zu bytes", lds);
   const int grid = (n + 16 * R - 1) / (16 * R);
-  gemm_skinny_kernel<MB, R, EPI, TO><<<grid, n_waves * 64, lds, s>>>(x, w, (TO*)c, m, n, k, k_per_wave);
+  gemm_skinny_kernel<MB, R, U, FAST, EPI, TO><<<grid, n_waves * 64, lds, s>>>(x, w, (TO*)c, m, n, k, k_per_wave);
   return 0;
+}
+
+// How K is dealt to the waves of a workgroup.  Fast path: K = 128 * T, n_waves divides T and
+// every wave gets a multiple of U stages.  Otherwise the checked path with up to 8 waves.
+template <int MB, int R, int EPI, typename TO>
+static int launch_skinny_u(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
+  constexpr int cost = R + MB;            // 16-byte registers per stage and j
+  constexpr int max_waves = (R * MB <= 4) ? 8 : 4;      // bounds the reduction buffer
+  if (k % 128 == 0) {
+    const int t = k / 128;
+    const int us[3] = {4, 2, 1};
+    for (int ui = 0; ui < 3; ++ui) {
+      const int u = g_tune_u ? g_tune_u : us[ui];
+      if (u == 4 && cost > 3) continue;
+      if (u == 2 && cost > 6) continue;
+      for (int nw = g_tune_waves ? g_tune_waves : max_waves; nw >= 1; --nw) {
+        if (t % nw != 0 || (t / nw) % u != 0) continue;
+        if (nw < 4 && t / nw > 8 && u != 1) break;      // too few waves: try a smaller U first
+        const int kpw = k / nw;
+        if (u == 4) return launch_skinny<MB, R, (cost <= 3 ? 4 : 1), true, EPI, TO>(x, w, c, m, n, k, nw, kpw, s);
+        if (u == 2) return launch_skinny<MB, R, (cost <= 6 ? 2 : 1), true, EPI, TO>(x, w, c, m, n, k, nw, kpw, s);
+        return launch_skinny<MB, R, 1, true, EPI, TO>(x, w, c, m, n, k, nw, kpw, s);
+      }
+    }
+  }
+  int n_waves = k / 256;
+  if (n_waves < 1) n_waves = 1;
+  if (n_waves > max_waves) n_waves = max_waves;
+  int k_per_wave = (k + n_waves - 1) / n_waves;
+  k_per_wave = (k_per_wave + 127) / 128 * 128;
+  return launch_skinny<MB, R, 1, false, EPI, TO>(x, w, c, m, n, k, n_waves, k_per_wave, s);
 }
 
 template <int EPI, typename TO>
@@ -155,9 +230,10 @@ static int dispatch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int
   int r = 1;
   if (n >= 32768) r = 4;
   else if (n >= 16384) r = 2;
+  if (g_tune_r) r = g_tune_r;
   if (EPI == 1 && r < 2) r = 2;
   if (mb >= 3 && r > 2) r = 2;
-#define RB_SK(MBV, RV) return launch_skinny<MBV, RV, EPI, TO>(x, w, c, m, n, k, s)
+#define RB_SK(MBV, RV) return launch_skinny_u<MBV, RV, EPI, TO>(x, w, c, m, n, k, s)
   if (mb == 1) {
     if (r == 4) RB_SK(1, 4);
     if (r == 2) RB_SK(1, 2);

@@ -48,6 +48,8 @@ class Engine:
         self.cache = Cache(model.cache_requests(), n_slots=self.max_batch, max_tokens=max_tokens,
                            dtype=self.dtype, device=self.device, readers=model.cache_readers())
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0}
+        self.use_graphs = bool(model.graph_safe)
+        self._graphs: Dict[int, Any] = {}
         from ..sampling import Sampler
         self.sampler = Sampler(self.lib, self.device)
 
@@ -171,9 +173,29 @@ class Engine:
 
     def decode_step(self, slots: Sequence[int], tokens: Sequence[int], temperatures=None, uniforms=None) -> list:
         """One token per sequence in, the next token per sequence out: a step and the
-        sampling of its logits."""
-        logits = self.step([(s, [t]) for s, t in zip(slots, tokens)], "last")
-        return self.sampler.sample(logits, temperatures, uniforms)
+        sampling of its logits, replayed as a HIP graph per batch size (see
+        decode_graph.py); `use_graphs = False` runs the same kernels launch by launch."""
+        slots = [int(s) for s in slots]
+        tokens = [int(t) for t in tokens]
+        vocab = self.spec.vocab_size
+        for s, t in zip(slots, tokens):
+            if not 0 <= t < vocab:
+                raise InferenceError(f"slot {s}: token id out of range ({t}, vocabulary {vocab})")
+            if self.cache.length(s) + 1 > self.max_seq_len:
+                raise InferenceError(f"slot {s}: sequence position >= max_seq ({self.max_seq_len})")
+        if not self.use_graphs:
+            logits = self.step([(s, [t]) for s, t in zip(slots, tokens)], "last")
+            return self.sampler.sample(logits, temperatures, uniforms)
+        from .decode_graph import DecodeGraph
+        n = len(slots)
+        if n not in self._graphs:
+            if len(self._graphs) >= 24:
+                self._graphs.pop(next(iter(self._graphs)))
+            self._graphs[n] = DecodeGraph(self, n)
+        out = self._graphs[n].run(slots, tokens, temperatures, uniforms)
+        self.stats["steps"] += 1
+        self.stats["decode_tokens"] += n
+        return out
 
     # ------------------------------------------------------------------ generation
     def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 256, temperature: float = 0.7,

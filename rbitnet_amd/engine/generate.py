@@ -13,7 +13,8 @@ runtime.rs:71 no step is run whose logits nobody reads: a sequence that has reac
 max_tokens does not feed its last token.
 
 `engine` needs: alloc_slot(), free_slot(slot), step(entries, want) -> logits,
-sampler.sample(logits, temperatures, uniforms) -> tokens, max_batch, max_seq_len,
+sampler.sample(logits, temperatures, uniforms) -> tokens, decode_step(slots, tokens,
+temperatures, uniforms) -> tokens, max_batch, max_seq_len,
 cache.n_pages / cache.kv_groups (for admission), spec.stop_token_ids.
 """
 from __future__ import annotations
@@ -108,30 +109,33 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 256, te
             running.append(_Running(index=i, slot=slot, budget=max_tokens,
                                     room=engine.max_seq_len - len(prompts[i]), result=results[i]))
         try:
-            feed = [(r.slot, prompts[r.index]) for r in running]
+            logits = engine.step([(r.slot, prompts[r.index]) for r in running], "last")
+            tokens = engine.sampler.sample(
+                logits, [temperature] * len(running),
+                [uniform(seed, r.index, 0) for r in running] if temperature > 0 else None)
             while running:
-                logits = engine.step(feed, "last")
-                temps = [temperature] * len(running)
-                us = [uniform(seed, r.index, len(r.result.tokens)) for r in running] if temperature > 0 else None
-                tokens = engine.sampler.sample(logits, temps, us)
                 survivors: List[_Running] = []
-                feed = []
+                feed: List[int] = []
                 for r, tok in zip(running, tokens):
-                    # pages: a sequence that cannot get another page ends here as well
                     verdict = decide(tok, len(r.result.tokens), max_tokens, r.room - 1, stop_ids)
                     if verdict != "stop":
                         r.result.tokens.append(int(tok))
                         r.room -= 1
+                    # a sequence that cannot get another page ends here as well
                     if verdict is None and not _has_page_for(engine, r.slot):
                         verdict = "context"
                     if verdict is None:
                         survivors.append(r)
-                        feed.append((r.slot, [int(tok)]))
+                        feed.append(int(tok))
                     else:
                         r.result.finish_reason = verdict
                         engine.free_slot(r.slot)
                         r.slot = -1
                 running = survivors
+                if running:
+                    tokens = engine.decode_step(
+                        [r.slot for r in running], feed, [temperature] * len(running),
+                        [uniform(seed, r.index, len(r.result.tokens)) for r in running] if temperature > 0 else None)
         finally:
             for r in running:
                 if r.slot >= 0:

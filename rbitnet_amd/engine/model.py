@@ -112,6 +112,11 @@ class Model:
                     f"which keeps only the last {theirs} positions")
         return out
 
+    @property
+    def graph_safe(self) -> bool:
+        return (all(getattr(b, "graph_safe", False) for b in self.blocks)
+                and getattr(self.final_norm, "graph_safe", False))
+
     def max_positions(self) -> int:
         return self.spec.max_positions
 

@@ -34,6 +34,8 @@ _MATRIX_CORE_HEAD_DIMS = (64, 128)
 
 
 class Attention(Part):
+    graph_safe = True
+
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env
         self.n_heads = int(params["num_heads"])

@@ -72,6 +72,11 @@ class CacheRequest:
 
 
 class Part:
+    # True when forward only launches kernels on the current stream (no host
+    # synchronisation, no host-side reads of device data): the decode step may then be
+    # captured into a HIP graph.  A part that does not say so is run launch by launch.
+    graph_safe = False
+
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {}
 

@@ -30,6 +30,10 @@ class PreNormBlock:
         self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, env)
         self.segments = dict(DEFAULT_SEGMENTS, **(getattr(layer_spec, "segments", None) or {}))
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(p, "graph_safe", False) for p in (self.norm1, self.mixer, self.norm2, self.feed_forward))
+
     def parts(self) -> Dict[str, object]:
         return {self.segments["norm1"]: self.norm1, self.segments["mixer"]: self.mixer,
                 self.segments["norm2"]: self.norm2, self.segments["feed_forward"]: self.feed_forward}

@@ -23,6 +23,8 @@ DEFAULT_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "do
 
 
 class SwiGLU(Part):
+    graph_safe = True
+
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env
         self.ff = int(params["intermediate_size"])

@@ -21,6 +21,8 @@ from .base import BuildEnv, Part, TensorSpec, register_norm
 
 
 class RMSNorm(Part):
+    graph_safe = True
+
     def __init__(self, params: Dict, env: BuildEnv):
         self.size = int(params["size"])
         self.eps = float(params["eps"])

@@ -50,6 +50,8 @@ def rope_inverse_frequencies(head_dim: int, theta: float, scaling: Optional[Dict
 
 
 class Rope(Part):
+    graph_safe = True
+
     def __init__(self, params: Dict, env: BuildEnv):
         self.head_dim = int(params["head_dim"])
         self.style = {"interleaved": 0, "half": 1}.get(params.get("style", "interleaved"))
@@ -72,6 +74,8 @@ class Rope(Part):
 
 
 class NoPosition(Part):
+    graph_safe = True
+
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env
         self.max_positions = int(params.get("max_positions", 1 << 30))

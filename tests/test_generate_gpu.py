@@ -167,3 +167,48 @@ def test_command_line_generate_and_inspect(tmp_path):
     ins = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "rbitnet"), "inspect", folder],
                          capture_output=True, text=True, env=env)
     assert ins.returncode == 0 and "tensors=21" in ins.stdout and "... and 1 more" in ins.stdout
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_decode_equals_launch_by_launch(dtype):
+    """The captured decode step against the same kernels launched one by one: the same
+    tokens and logits on every replay, with eager work and synchronisations in between,
+    across a page boundary, and for a batch that shrinks."""
+    name = "C"
+    eng_g = _engine(name, dtype, max_batch=3)
+    eng_e = _engine(name, dtype, max_batch=3)
+    eng_e.use_graphs = False
+    assert eng_g.use_graphs
+    prompts = [tokens_for(name, n, 30 + i) for i, n in enumerate([60, 5, 130])]
+    outs = []
+    for eng in (eng_g, eng_e):
+        slots = [eng.alloc_slot() for _ in prompts]
+        logits = eng.step(list(zip(slots, prompts)), "last")
+        toks = eng.sampler.sample(logits)
+        hist = [list(toks)]
+        for step in range(12):
+            if step == 8:                       # the shortest request leaves
+                eng.free_slot(slots.pop(1))
+                toks.pop(1)
+            temps = [0.0, 0.9, 0.0][:len(slots)]
+            us = [0.1 * (step % 7), 0.37, 0.5][:len(slots)]
+            toks = eng.decode_step(slots, toks, temps, us)
+            hist.append(list(toks))
+            if eng.use_graphs:
+                g = eng._graphs[len(slots)]
+                hist.append(g.logits.float().cpu().clone())
+                torch.cuda.synchronize()
+                _ = (torch.ones(1000, device="cuda") * 2).sum().item()      # unrelated eager work
+            else:
+                hist.append(None)
+        outs.append(hist)
+        for s in slots:
+            eng.free_slot(s)
+        eng.cache.check()
+    tok_g = [h for h in outs[0] if isinstance(h, list)]
+    tok_e = [h for h in outs[1] if isinstance(h, list)]
+    assert tok_g == tok_e
+    # and the graph's logits against the plain implementation at the last step
+    seq0 = prompts[0] + [t[0] for t in tok_g[:-1]]
+    last = [h for h in outs[0] if isinstance(h, torch.Tensor)][-1]
+    assert max_err(last[0:1], plain_logits(name, tuple(seq0))[-1:]) < TOL[dtype]

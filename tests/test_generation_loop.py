@@ -45,6 +45,9 @@ class ScriptedEngine:
     def sample(self, logits, temperatures=None, uniforms=None):
         return list(logits)
 
+    def decode_step(self, slots, tokens, temperatures=None, uniforms=None):
+        return self.sample(self.step([(s, [t]) for s, t in zip(slots, tokens)], "last"))
+
 
 def test_decide():
     assert decide(9, 0, 10, 5, {9}) == "stop"
