@@ -191,27 +191,19 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int n
   return 0;
 }
 
-// How K is dealt to the waves of a workgroup.  Fast path: K = 128 * T, n_waves divides T and
-// every wave gets a multiple of U stages.  Otherwise the checked path with up to 8 waves.
+// How K is dealt to the waves of a workgroup.  Fast path: K = 128 * T and the wave count
+// divides T.  Otherwise the checked path with up to 8 waves.  Measured on the Llama-3-8B
+// products at M = 1..8: one stage in flight per wave (U = 1) is as fast as 2 or 4, and 4
+// waves beat 8 at K = 4096, 8 beat 4 at K = 14336.
 template <int MB, int R, int EPI, typename TO>
 static int launch_skinny_u(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
-  constexpr int cost = R + MB;            // 16-byte registers per stage and j
   constexpr int max_waves = (R * MB <= 4) ? 8 : 4;      // bounds the reduction buffer
   if (k % 128 == 0) {
     const int t = k / 128;
-    const int us[3] = {4, 2, 1};
-    for (int ui = 0; ui < 3; ++ui) {
-      const int u = g_tune_u ? g_tune_u : us[ui];
-      if (u == 4 && cost > 3) continue;
-      if (u == 2 && cost > 6) continue;
-      for (int nw = g_tune_waves ? g_tune_waves : max_waves; nw >= 1; --nw) {
-        if (t % nw != 0 || (t / nw) % u != 0) continue;
-        if (nw < 4 && t / nw > 8 && u != 1) break;      // too few waves: try a smaller U first
-        const int kpw = k / nw;
-        if (u == 4) return launch_skinny<MB, R, (cost <= 3 ? 4 : 1), true, EPI, TO>(x, w, c, m, n, k, nw, kpw, s);
-        if (u == 2) return launch_skinny<MB, R, (cost <= 6 ? 2 : 1), true, EPI, TO>(x, w, c, m, n, k, nw, kpw, s);
-        return launch_skinny<MB, R, 1, true, EPI, TO>(x, w, c, m, n, k, nw, kpw, s);
-      }
+    const int first_nw = k >= 8192 ? max_waves : 4;
+    for (int nw = g_tune_waves ? g_tune_waves : first_nw; nw >= 1; --nw) {
+      if (t % nw != 0) continue;
+      return launch_skinny<MB, R, 1, true, EPI, TO>(x, w, c, m, n, k, nw, k / nw, s);
     }
   }
   int n_waves = k / 256;
@@ -228,8 +220,8 @@ static int dispatch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int
   // rows of W per wave: more of them reuse the token operand better, fewer give more
   // workgroups; keep at least about two workgroups per compute unit
   int r = 1;
-  if (n >= 32768) r = 4;
-  else if (n >= 16384) r = 2;
+  if (n >= 16384) r = 4;
+  else if (n >= 6144) r = 2;
   if (g_tune_r) r = g_tune_r;
   if (EPI == 1 && r < 2) r = 2;
   if (mb >= 3 && r > 2) r = 2;
@@ -251,6 +243,172 @@ static int dispatch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int
   }
 #undef RB_SK
   RB_REQUIRE(false, "rb_gemm_bf16: internal: no skinny kernel for M=%d R=%d", m, r);
+}
+
+// =============================================================================== skinny, tokens resident
+// The same product for M <= 64 with the token operand held in registers: a wave owns a
+// fixed slice of K (32 * XQ values), loads the tokens' fragments for it once, and then
+// streams the W rows of one 16-row tile after the other through the matrix cores, the
+// next tile's loads in flight while the current one is multiplied.  Inside the loop W is
+// the only thing read from memory.  A workgroup's waves cover adjacent K slices and add
+// their sums through LDS.
+template <int MB, int XQ, int EPI, typename TO>
+__global__ __launch_bounds__(512) void gemm_resident_kernel(const bf16_t* __restrict__ x,
+                                                             const bf16_t* __restrict__ w, TO* __restrict__ c,
+                                                             int m, int n, int k, int tiles_per_wg) {
+  extern __shared__ float red[];      // [2][waves - 1][MB * 4][64]
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n_waves = blockDim.x >> 6;
+  const int r = lane & 15;
+  const int kq = lane >> 4;
+  const int n_tiles = (n + 15) / 16;
+  const int tile0 = blockIdx.x * tiles_per_wg;
+  int t_count = n_tiles - tile0;
+  if (t_count > tiles_per_wg) t_count = tiles_per_wg;
+  const int k0 = (blockIdx.y * n_waves + wave) * (32 * XQ) + 8 * kq;
+  TO* cpart = c + (size_t)blockIdx.y * m * (EPI == 1 ? n / 2 : n);
+
+  // ---- the tokens' fragments for this wave's slice of K
+  Frag8 b[XQ][MB];
+#pragma unroll
+  for (int cb = 0; cb < MB; ++cb) {
+    const int row = 16 * cb + r;
+    const bf16_t* xrow = x + (size_t)(row < m ? row : 0) * k + k0;
+#pragma unroll
+    for (int j = 0; j < XQ; ++j) b[j][cb].u = load16(xrow + 32 * j);
+  }
+
+  Frag8 a0[XQ], a1[XQ];
+  auto load_tile = [&](Frag8* a, int t) {
+    int row = (tile0 + t) * 16 + r;
+    if (row >= n) row = 0;                       // results of such rows are never stored
+    const bf16_t* wrow = w + (size_t)row * k + k0;
+#pragma unroll
+    for (int j = 0; j < XQ; ++j) a[j].u = load16(wrow + 32 * j);
+  };
+  f32x4_t gate[MB];                              // EPI 1: the gate tile's sums wait for the up tile
+  auto finish_tile = [&](const Frag8* a, int t) {
+    f32x4_t acc[MB];
+#pragma unroll
+    for (int cb = 0; cb < MB; ++cb) acc[cb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < XQ; ++j)
+#pragma unroll
+      for (int cb = 0; cb < MB; ++cb) acc[cb] = mfma16(a[j], b[j][cb], acc[cb]);
+    // the wave that gathers this tile's sums: tiles of a gate/up pair go to the same one
+    const int owner = (EPI == 1 ? (t >> 1) : t) % n_waves;
+    if (n_waves > 1) {
+      float* buf = red + (size_t)(t & 1) * (n_waves - 1) * MB * 4 * 64;
+      if (wave != owner) {
+        const int slot = wave < owner ? wave : wave - 1;
+        float* dst = buf + (size_t)slot * MB * 4 * 64 + lane;
+#pragma unroll
+        for (int cb = 0; cb < MB; ++cb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dst[(cb * 4 + i) * 64] = acc[cb][i];
+      }
+      __syncthreads();
+      if (wave == owner) {
+        for (int ww = 0; ww < n_waves - 1; ++ww) {
+          const float* src = buf + (size_t)ww * MB * 4 * 64 + lane;
+#pragma unroll
+          for (int cb = 0; cb < MB; ++cb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[cb][i] += src[(cb * 4 + i) * 64];
+        }
+      }
+    }
+    if (wave != owner) return;
+    const int tile = tile0 + t;
+    if (EPI == 0) {
+#pragma unroll
+      for (int cb = 0; cb < MB; ++cb) {
+        const int mm = 16 * cb + r;
+        const int nn = tile * 16 + 4 * kq;
+        if (mm >= m) continue;
+        TO* dst = cpart + (size_t)mm * n + nn;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nn + i < n) Num<TO>::store(dst + i, acc[cb][i]);
+      }
+    } else if ((t & 1) == 0) {
+#pragma unroll
+      for (int cb = 0; cb < MB; ++cb) gate[cb] = acc[cb];
+    } else {
+      const int half_n = n / 2;
+#pragma unroll
+      for (int cb = 0; cb < MB; ++cb) {
+        const int mm = 16 * cb + r;
+        const int nn = (tile >> 1) * 16 + 4 * kq;
+        if (mm >= m) continue;
+        TO* dst = cpart + (size_t)mm * half_n + nn;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nn + i < half_n) Num<TO>::store(dst + i, silu_f32(gate[cb][i]) * acc[cb][i]);
+      }
+    }
+  };
+
+  if (t_count <= 0) return;
+  load_tile(a0, 0);
+  int t = 0;
+  for (; t + 2 < t_count; t += 2) {              // tiles t + 1 and t + 2 exist: loads are unconditional
+    load_tile(a1, t + 1);
+    finish_tile(a0, t);
+    load_tile(a0, t + 2);
+    finish_tile(a1, t + 1);
+  }
+  if (t + 1 < t_count) {
+    load_tile(a1, t + 1);
+    finish_tile(a0, t);
+    finish_tile(a1, t + 1);
+  } else {
+    finish_tile(a0, t);
+  }
+}
+
+static int g_res_tiles = 0;
+extern "C" void rb_tune_resident(int waves, int parts, int tiles) {      // experiments only; 0 = built-in
+  (void)waves;
+  (void)parts;
+  g_res_tiles = tiles;
+}
+
+template <int MB, int XQ, int EPI, typename TO>
+static int launch_resident(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, int parts,
+                           hipStream_t s) {
+  const int slices = k / (32 * XQ);
+  const int n_waves = slices / parts;
+  const int n_tiles = (n + 15) / 16;
+  // tiles per workgroup: as many as leave about one workgroup per compute unit (measured on
+  // the 28672 x 4096 and 128256 x 4096 products: 224 and 501 workgroups beat 448 and 1002)
+  int tiles = g_res_tiles ? g_res_tiles : 16;
+  while (!g_res_tiles && tiles > 2 && (long long)((n_tiles + tiles - 1) / tiles) * parts < 200) tiles >>= 1;
+  if (EPI == 1 && (tiles & 1)) tiles += 1;
+  const size_t lds = (size_t)2 * (n_waves > 1 ? n_waves - 1 : 0) * MB * 4 * 64 * sizeof(float);
+  dim3 grid((n_tiles + tiles - 1) / tiles, parts);
+  gemm_resident_kernel<MB, XQ, EPI, TO><<<grid, n_waves * 64, lds, s>>>(x, w, (TO*)c, m, n, k, tiles);
+  return 0;
+}
+
+// true if the resident kernel takes these sizes
+template <int EPI, typename TO>
+static bool try_resident(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, int parts, hipStream_t s,
+                         int* rc) {
+  const int mb = (m + 15) / 16;
+  const int xq = mb == 1 ? 16 : (mb == 2 ? 8 : 4);
+  if (k % (32 * xq) != 0) return false;
+  const int slices = k / (32 * xq);
+  if (parts < 1 || slices % parts != 0) return false;
+  const int n_waves = slices / parts;
+  if (n_waves > 8) return false;
+  if (EPI == 1 && (n % 32 != 0)) return false;
+  if (mb == 1) *rc = launch_resident<1, 16, EPI, TO>(x, w, c, m, n, k, parts, s);
+  else if (mb == 2) *rc = launch_resident<2, 8, EPI, TO>(x, w, c, m, n, k, parts, s);
+  else if (mb == 3) *rc = launch_resident<3, 4, EPI, TO>(x, w, c, m, n, k, parts, s);
+  else *rc = launch_resident<4, 4, EPI, TO>(x, w, c, m, n, k, parts, s);
+  return true;
 }
 
 // =============================================================================== tiled
@@ -397,6 +555,9 @@ static int launch_tiled(const bf16_t* x, const bf16_t* w, void* c, int m, int n,
   return 0;
 }
 
+static int g_use_resident = 1;
+extern "C" void rb_tune_use_resident(int on) { g_use_resident = on; }
+
 extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out, int epilogue, int m, int n,
                             int k, void* stream) {
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_bf16: bad sizes M=%d N=%d K=%d", m, n, k);
@@ -408,14 +569,26 @@ extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* xa = (const bf16_t*)a;
   const bf16_t* wa = (const bf16_t*)w;
-  int rc;
+  int rc = 0;
   if (m <= 64) {
-    if (epilogue == 0)
-      rc = dtype_out == RB_F32 ? dispatch_skinny<0, float>(xa, wa, c, m, n, k, s)
-                               : dispatch_skinny<0, bf16_t>(xa, wa, c, m, n, k, s);
-    else
-      rc = dtype_out == RB_F32 ? dispatch_skinny<1, float>(xa, wa, c, m, n, k, s)
-                               : dispatch_skinny<1, bf16_t>(xa, wa, c, m, n, k, s);
+    bool done = false;
+    // many rows of W and at most 16 tokens: the kernel that keeps the tokens in registers
+    if (g_use_resident && m <= 16 && n > 8192) {
+      if (epilogue == 0)
+        done = dtype_out == RB_F32 ? try_resident<0, float>(xa, wa, c, m, n, k, 1, s, &rc)
+                                   : try_resident<0, bf16_t>(xa, wa, c, m, n, k, 1, s, &rc);
+      else
+        done = dtype_out == RB_F32 ? try_resident<1, float>(xa, wa, c, m, n, k, 1, s, &rc)
+                                   : try_resident<1, bf16_t>(xa, wa, c, m, n, k, 1, s, &rc);
+    }
+    if (!done) {
+      if (epilogue == 0)
+        rc = dtype_out == RB_F32 ? dispatch_skinny<0, float>(xa, wa, c, m, n, k, s)
+                                 : dispatch_skinny<0, bf16_t>(xa, wa, c, m, n, k, s);
+      else
+        rc = dtype_out == RB_F32 ? dispatch_skinny<1, float>(xa, wa, c, m, n, k, s)
+                                 : dispatch_skinny<1, bf16_t>(xa, wa, c, m, n, k, s);
+    }
   } else {
     if (epilogue == 0)
       rc = dtype_out == RB_F32 ? launch_tiled<0, float>(xa, wa, c, m, n, k, s)
