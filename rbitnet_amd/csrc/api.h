@@ -74,6 +74,14 @@ int rb_attention_decode_bf16(const void* q, const void* k_pages, const void* v_p
                              int n_heads, int n_kv_heads, int head_dim, float scale, int window, int n_splits,
                              float* workspace, void* stream);
 
+//   decode, fused: rotation of q and the new k, cache write and attention in one kernel (plus the
+//   combination of the splits when there are several).  qkv float32 [B, (Hq + 2 Hk) D] as for
+//   rb_rope_kv_write.
+int rb_attention_decode_fused_bf16(const float* qkv, const float* cos, const float* sin, int style, void* k_pages,
+                                   void* v_pages, void* out, const int32_t* tok_pos, const int32_t* block_table,
+                                   int bt_stride, int n_seqs, int n_heads, int n_kv_heads, int head_dim, float scale,
+                                   int window, int n_splits, float* workspace, void* stream);
+
 // tokens[r] = argmax of logits[r, :] (NaN counts as -inf, lowest index among equals), or, where
 // temperature[r] > 0, the first index whose running sum of exp(z/T - max) reaches u[r] times the total.
 int rb_sample(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,

@@ -68,6 +68,8 @@ class Kernels:
             "rb_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_prefill_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_decode_bf16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
+            "rb_attention_decode_fused_bf16": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
+                                               _P, _P],
             "rb_sample": [_P, _I, _I, _P, _P, _P, _P],
         }
         for name, args in sig.items():
@@ -213,6 +215,30 @@ class Kernels:
                                                     _ptr(block_table), block_table.shape[1], n, n_heads, n_kv,
                                                     head_dim, float(scale), int(window or 0), int(n_splits),
                                                     _ptr(workspace), self._stream()))
+
+    def attention_decode_fused_bf16(self, qkv, cos, sin, style, k_pages, v_pages, out, tok_pos, block_table,
+                                    n_heads, n_kv, head_dim, scale, window, n_splits, workspace) -> None:
+        n = qkv.shape[0]
+        _check(qkv, "qkv", torch.float32, (n, (n_heads + 2 * n_kv) * head_dim))
+        if cos is not None:
+            _check(cos, "cos", torch.float32)
+            _check(sin, "sin", torch.float32, cos.shape)
+            if cos.shape[1] != head_dim // 2:
+                raise KernelError("angle table width mismatch")
+        _check(k_pages, "k_pages", torch.bfloat16)
+        _check(v_pages, "v_pages", torch.bfloat16, k_pages.shape)
+        if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, head_dim):
+            raise KernelError("cache pages do not match the head counts")
+        _check(out, "out", torch.bfloat16, (n, n_heads * head_dim))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(block_table, "block_table", torch.int32)
+        _check(workspace, "workspace", torch.float32)
+        if workspace.numel() < n * n_heads * n_splits * (head_dim + 2):
+            raise KernelError("decode attention workspace too small")
+        self._ok(self._lib.rb_attention_decode_fused_bf16(
+            _ptr(qkv), _ptr(cos), _ptr(sin), int(style), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tok_pos),
+            _ptr(block_table), block_table.shape[1], n, n_heads, n_kv, head_dim, float(scale), int(window or 0),
+            int(n_splits), _ptr(workspace), self._stream()))
 
     def sample(self, logits: torch.Tensor, temperature: Optional[torch.Tensor], u: Optional[torch.Tensor],
                tokens: torch.Tensor) -> None:

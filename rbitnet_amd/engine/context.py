@@ -63,12 +63,12 @@ class StepContext:
         self.block_tables: Dict[int, torch.Tensor] = {}
         for key, width in tables:
             self.block_tables[key] = take(b * width).view(b, width)
-        self._workspaces: Dict[Tuple[int, int], Tuple[int, torch.Tensor]] = {}
+        self._workspaces: Dict[Tuple[int, int, int], Tuple] = {}
 
-    def decode_workspace(self, n_heads: int, head_dim: int, n_kv_heads: int = 1) -> Tuple[int, torch.Tensor]:
+    def decode_workspace(self, n_heads: int, head_dim: int, n_kv_heads: int = 1) -> Tuple:
         """Split count and scratch for decode attention: enough workgroups to fill the
         GPU, whatever the context length (each split strides over the pages)."""
-        key = (n_heads, head_dim)
+        key = (n_heads, head_dim, n_kv_heads)
         if key not in self._workspaces:
             n_splits = max(1, min(32, 2048 // max(1, self.n_seqs * n_heads)))
             ws = torch.empty(self.n_seqs * n_heads * n_splits * (head_dim + 2), dtype=torch.float32,

@@ -69,10 +69,10 @@ class _StaticContext:
         self.host_slots: List[int] = [0] * b
         self.host_past: List[int] = [0] * b
         self.max_kv_len = 0
-        self._workspaces: Dict[Tuple[int, int], Tuple[int, torch.Tensor]] = {}
+        self._workspaces: Dict[Tuple[int, int, int], Tuple] = {}
 
     def decode_workspace(self, n_heads: int, head_dim: int, n_kv_heads: int = 1):
-        key = (n_heads, head_dim)
+        key = (n_heads, head_dim, n_kv_heads)
         if key not in self._workspaces:
             n_splits = max(1, min(32, 2048 // max(1, self.n_seqs * n_heads)))
             ws = torch.empty(self.n_seqs * n_heads * n_splits * (head_dim + 2), dtype=torch.float32,

@@ -31,6 +31,7 @@ from .linear import linear
 
 DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight"}
 _MATRIX_CORE_HEAD_DIMS = (64, 128)
+_DECODE_GROUPS = (1, 2, 4, 8)           # query heads per kv head the decode kernels are built for
 
 
 class Attention(Part):
@@ -88,18 +89,27 @@ class Attention(Part):
         hq, hk, d = self.n_heads, self.n_kv, self.head_dim
         owns = self.cache_from is None
         qkv = linear(lib, h, self.w_qkv, torch.float32)
-        q = torch.empty((t, hq, d), dtype=self.env.dtype, device=h.device)
         bt = view.block_table
-        if owns:
-            self.position.encode_and_store(qkv, q, view.k_pages, view.v_pages, ctx, bt, hq, hk, d)
-        else:
-            self.position.encode_and_store(qkv, q, None, None, ctx, bt, hq, 0, d)
         attn = torch.empty((t, hq * d), dtype=self.env.dtype, device=h.device)
         window = int(self.window) if self.window is not None else 0
         fast = (self.env.dtype == torch.bfloat16 and d in _MATRIX_CORE_HEAD_DIMS
                 and not getattr(self.env, "generic_only", False))
-        if fast and ctx.max_q_len == 1:
-            n_splits, workspace = ctx.decode_workspace(hq, d)
+        decode = fast and ctx.max_q_len == 1 and (hq // hk) in _DECODE_GROUPS
+        tables = getattr(self.position, "rotation_tables", None)
+        if decode and owns and tables is not None:
+            # one kernel: rotation, cache write, attention over the pages
+            cos, sin, style = tables()
+            n_splits, workspace = ctx.decode_workspace(hq, d, hk)
+            lib.attention_decode_fused_bf16(qkv, cos, sin, style, view.k_pages, view.v_pages, attn, ctx.tok_pos, bt,
+                                            hq, hk, d, self.scale, window, n_splits, workspace)
+            return linear(lib, attn, self.w_o, torch.float32)
+        q = torch.empty((t, hq, d), dtype=self.env.dtype, device=h.device)
+        if owns:
+            self.position.encode_and_store(qkv, q, view.k_pages, view.v_pages, ctx, bt, hq, hk, d)
+        else:
+            self.position.encode_and_store(qkv, q, None, None, ctx, bt, hq, 0, d)
+        if decode:
+            n_splits, workspace = ctx.decode_workspace(hq, d, hk)
             lib.attention_decode_bf16(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, bt, hq, hk, d,
                                       self.scale, window, n_splits, workspace)
         elif fast:

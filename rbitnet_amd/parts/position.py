@@ -3,6 +3,8 @@ rotated q and writes k and v into the cache, keyed by each token's absolute posi
 
 Interface: encode_and_store(qkv, q_out, k_pages, v_pages, ctx, block_table,
                             n_heads, n_kv_heads, head_dim)
+Optional:  rotation_tables() -> (cos, sin, style) when the encoding is a per-position,
+           per-pair rotation; a mixer may then apply it inside a fused kernel.
 
 "rope": the rotation of the reference (crates/bitnet-core/src/llama/model.rs:122-136):
 inv_i = 1 / theta^(2i/D), angle = pos * inv_i, pairs (x[2i], x[2i+1]) ("interleaved") or
@@ -68,6 +70,10 @@ class Rope(Part):
             self.cos = torch.cos(angles).to(torch.float32).to(env.device).contiguous()
             self.sin = torch.sin(angles).to(torch.float32).to(env.device).contiguous()
 
+    def rotation_tables(self):
+        """(cos, sin, pairing style): lets a mixer fold the rotation into its own kernel."""
+        return self.cos, self.sin, self.style
+
     def encode_and_store(self, qkv, q_out, k_pages, v_pages, ctx, block_table, n_heads, n_kv, head_dim) -> None:
         self.env.lib.rope_kv_write(qkv, self.cos, self.sin, self.style, q_out, k_pages, v_pages, ctx.tok_pos,
                                    ctx.tok_seq, block_table, n_heads, n_kv, head_dim)
@@ -79,6 +85,9 @@ class NoPosition(Part):
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env
         self.max_positions = int(params.get("max_positions", 1 << 30))
+
+    def rotation_tables(self):
+        return None, None, 0
 
     def encode_and_store(self, qkv, q_out, k_pages, v_pages, ctx, block_table, n_heads, n_kv, head_dim) -> None:
         self.env.lib.rope_kv_write(qkv, None, None, 0, q_out, k_pages, v_pages, ctx.tok_pos, ctx.tok_seq,

@@ -320,3 +320,49 @@ def test_sample_greedy_and_inverse_cdf(lib):
     for r in range(7):
         row = torch.nan_to_num(logits[r], nan=-float("inf"))
         assert tokens[r].item() == sample_token(row, float(temps[r]), float(us[r])), r
+
+
+@pytest.mark.parametrize("style", [0, 1])
+@pytest.mark.parametrize("n_heads,n_kv,d,window,n_splits", [(4, 1, 128, 0, 3), (8, 8, 64, 0, 1), (8, 4, 128, 0, 8),
+                                                           (8, 1, 64, 90, 2), (2, 2, 128, 65, 5), (4, 2, 64, 0, 32)])
+def test_attention_decode_fused_bf16(lib, n_heads, n_kv, d, window, n_splits, style):
+    """Rotation, cache write and attention in one kernel (and the combination of splits),
+    against the separate steps computed plainly; called three times in a row."""
+    past, q_lens = [0, 70, 129, 63, 64, 300], [1, 1, 1, 1, 1, 1]
+    dtype = torch.bfloat16
+    nb = len(past)
+    g, bt, tok_seq, tok_pos, total = _paged_setup(past, q_lens, n_kv, d, dtype, seed=n_heads + 5)
+    k_past = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in past]
+    v_past = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in past]
+    inv = 1.0 / (10000.0 ** (torch.arange(d // 2).double() * 2 / d))
+    ang = torch.arange(400).double()[:, None] * inv[None]
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    scale = 1 / math.sqrt(d)
+    ws = torch.full((nb * n_heads * n_splits * (d + 2),), float("nan"), device=DEV)
+    for call in range(3):
+        qkv = torch.randn(nb, (n_heads + 2 * n_kv) * d, generator=g) * 1.5
+        # plain: rotate q and k, round to bfloat16, append k and v, attend
+        rot = torch.empty(nb, n_heads + n_kv, d, dtype=torch.float64)
+        for b in range(nb):
+            heads = qkv[b].double().view(n_heads + 2 * n_kv, d)[:n_heads + n_kv]
+            z = torch.polar(torch.ones(d // 2, dtype=torch.float64), ang[past[b]])
+            if style == 0:
+                rot[b] = torch.view_as_real(torch.view_as_complex(heads.reshape(-1, d // 2, 2)) * z).reshape(-1, d)
+            else:
+                c = torch.complex(heads[:, :d // 2], heads[:, d // 2:]) * z
+                rot[b] = torch.cat([c.real, c.imag], dim=1)
+        q = rot[:, :n_heads].to(dtype)
+        k_new = rot[:, n_heads:].to(dtype)
+        v_new = qkv.view(nb, n_heads + 2 * n_kv, d)[:, n_heads + n_kv:].to(dtype)
+        k_full = [torch.cat([k_past[b], k_new[b:b + 1]]) for b in range(nb)]
+        v_full = [torch.cat([v_past[b], v_new[b:b + 1]]) for b in range(nb)]
+        want = _attention_ref(q, k_full, v_full, tok_seq, tok_pos, n_heads, n_kv, scale, window)
+        kp, vp = _fill_pages(k_past, v_past, bt, 64, n_kv, d, dtype)       # the new position holds NaN
+        kp, vp = kp.to(DEV), vp.to(DEV)
+        out = torch.full((nb, n_heads * d), float("nan"), dtype=dtype, device=DEV)
+        lib.attention_decode_fused_bf16(qkv.to(DEV), cos, sin, style, kp, vp, out, tok_pos.to(DEV), bt.to(DEV),
+                                        n_heads, n_kv, d, scale, window, n_splits, ws)
+        assert _rel(out, want) < 1e-2, call
+        for b in range(nb):
+            page, off = int(bt[b, past[b] // 64]), past[b] % 64
+            assert torch.equal(kp[page, :, off].cpu(), k_new[b]) and torch.equal(vp[page, :, off].cpu(), v_new[b])
