@@ -84,8 +84,10 @@ int rb_attention_decode_fused_bf16(const float* qkv, const float* cos, const flo
 
 // tokens[r] = argmax of logits[r, :] (NaN counts as -inf, lowest index among equals), or, where
 // temperature[r] > 0, the first index whose running sum of exp(z/T - max) reaches u[r] times the total.
+// workspace: rb_sample_workspace_bytes(n_rows, vocab) bytes, 8-byte aligned, contents do not matter.
+int rb_sample_workspace_bytes(int n_rows, int vocab);
 int rb_sample(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,
-              int32_t* tokens, void* stream);
+              int32_t* tokens, void* workspace, void* stream);
 
 #ifdef __cplusplus
 }

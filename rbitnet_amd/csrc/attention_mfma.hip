@@ -268,163 +268,31 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
 }
 
 // =============================================================================== decode
-template <int D, int G>
+// One query per sequence.  A workgroup takes one kv head of one sequence (and one of n_splits
+// shares of its pages); each of its 4 waves walks its own pages, 64 keys at a time, with a
+// running softmax for the G query heads of the kv head, and the waves' states are merged
+// through LDS at the end.  No barrier inside the page loop: a page's 32 loads per lane are
+// all issued before the first is used, and four pages are in flight per workgroup.
+//
+// FUSED: q, k, v come straight from the projection (float32): q and the new k are rotated
+// here (angles from the table) and rounded through bfloat16 exactly as rope_kv_write_kernel
+// does, the new k and v are stored in the cache by the workgroup that owns the last page,
+// and where the loop reaches the token's own position it takes them from LDS, so that no
+// workgroup reads what another has just written.  Otherwise q is read as bfloat16 and the
+// cache already holds the token's key and value.
+//
+// With one split the result is written directly; with more, partial states go to the
+// workspace and attn_decode_combine_kernel adds them.  (Combining inside this kernel by a
+// ticket counter was tried: the device-scope fences it needs write back and invalidate the
+// L2 of every XCD and cost far more than the launch they save.)
+template <int D, int G, bool FUSED>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const float* __restrict__ qkv, const bf16_t* __restrict__ q_in, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int style, bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
     int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws) {
   constexpr int DL = D / 64;          // output elements per lane
   constexpr int QC = D / 32;          // 16-byte chunks of a quarter row of K
-  __shared__ float q_s[G][D];
-  __shared__ float p_s[4][G][16];
-  __shared__ float red_m[4][G], red_l[4][G];
-  __shared__ float red_acc[4][G][D];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
-  const int pos = tok_pos[b];
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int first_page = lo / RB_PAGE, last_page = pos / RB_PAGE;
-
-  for (int idx = tid; idx < G * D; idx += 256) {
-    const int gg = idx / D, d = idx % D;
-    q_s[gg][d] = bf16_to_f32(q[((size_t)b * n_heads + kvh * G + gg) * D + d]) * scale_log2;
-  }
-  __syncthreads();
-
-  float m_run[G], l_run[G], acc[G][DL];
-#pragma unroll
-  for (int gg = 0; gg < G; ++gg) {
-    m_run[gg] = -INFINITY;
-    l_run[gg] = 0.f;
-#pragma unroll
-    for (int e = 0; e < DL; ++e) acc[gg][e] = 0.f;
-  }
-  const int j = lane >> 2, part = lane & 3;
-  for (int pg = first_page + split; pg <= last_page; pg += n_splits) {
-    const int page = block_table[(size_t)b * bt_stride + pg];
-    const size_t base = ((size_t)page * n_kv + kvh) * RB_PAGE * D;
-    const int key0 = pg * RB_PAGE + wave * 16;
-    const int key = key0 + j;
-    const bool valid = key >= lo && key <= pos;
-    // ---- scores: lane (j, part) takes a quarter of key j's row
-    float s[G];
-#pragma unroll
-    for (int gg = 0; gg < G; ++gg) s[gg] = 0.f;
-    const bf16_t* krow = k_pages + base + (size_t)(wave * 16 + j) * D + part * (D / 4);
-#pragma unroll
-    for (int cidx = 0; cidx < QC; ++cidx) {
-      const uint4 u = load16(krow + cidx * 8);
-      const uint32_t wds[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float k0 = bf16_bits_to_f32(wds[e] & 0xffffu);
-        const float k1 = bf16_bits_to_f32(wds[e] >> 16);
-        const int d = part * (D / 4) + cidx * 8 + 2 * e;
-#pragma unroll
-        for (int gg = 0; gg < G; ++gg) s[gg] = fmaf(k1, q_s[gg][d + 1], fmaf(k0, q_s[gg][d], s[gg]));
-      }
-    }
-#pragma unroll
-    for (int gg = 0; gg < G; ++gg) {
-      float v = s[gg];
-      v += __shfl_xor(v, 1, 64);
-      v += __shfl_xor(v, 2, 64);
-      if (!valid) v = -INFINITY;
-      float mx = v;
-#pragma unroll
-      for (int o = 4; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-      const float m_new = fmaxf(m_run[gg], mx);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float corr = exp2f(m_run[gg] - m_safe);
-      const float p = exp2f(v - m_safe);
-      float ps = p;
-#pragma unroll
-      for (int o = 4; o < 64; o <<= 1) ps += __shfl_xor(ps, o, 64);
-      l_run[gg] = l_run[gg] * corr + ps;
-      m_run[gg] = m_new;
-#pragma unroll
-      for (int e = 0; e < DL; ++e) acc[gg][e] *= corr;
-      if (part == 0) p_s[wave][gg][j] = p;
-    }
-    __syncthreads();
-    // ---- weighted sum of the values: lane takes DL consecutive d
-    int jj_lo = lo - key0;
-    if (jj_lo < 0) jj_lo = 0;
-    int jj_hi = pos - key0;
-    if (jj_hi > 15) jj_hi = 15;
-    const bf16_t* vcol = v_pages + base + (size_t)(wave * 16) * D + lane * DL;
-    for (int jj = jj_lo; jj <= jj_hi; ++jj) {
-      float v[DL];
-      if (DL == 2) {
-        const uint32_t u = *reinterpret_cast<const uint32_t*>(vcol + (size_t)jj * D);
-        v[0] = bf16_bits_to_f32(u & 0xffffu);
-        v[DL - 1] = bf16_bits_to_f32(u >> 16);
-      } else {
-        v[0] = bf16_to_f32(vcol[(size_t)jj * D]);
-      }
-#pragma unroll
-      for (int gg = 0; gg < G; ++gg) {
-        const float p = p_s[wave][gg][jj];
-#pragma unroll
-        for (int e = 0; e < DL; ++e) acc[gg][e] = fmaf(p, v[e], acc[gg][e]);
-      }
-    }
-    __syncthreads();
-  }
-
-  // ---- combine the four waves, write this split's partial result
-#pragma unroll
-  for (int gg = 0; gg < G; ++gg) {
-    if (lane == 0) {
-      red_m[wave][gg] = m_run[gg];
-      red_l[wave][gg] = l_run[gg];
-    }
-#pragma unroll
-    for (int e = 0; e < DL; ++e) red_acc[wave][gg][lane * DL + e] = acc[gg][e];
-  }
-  __syncthreads();
-  for (int idx = tid; idx < G * D; idx += 256) {
-    const int gg = idx / D, d = idx % D;
-    float mx = red_m[0][gg];
-#pragma unroll
-    for (int w = 1; w < 4; ++w) mx = fmaxf(mx, red_m[w][gg]);
-    const float m_safe = (mx == -INFINITY) ? 0.f : mx;
-    float a = 0.f, l = 0.f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float f = exp2f(red_m[w][gg] - m_safe);
-      a += red_acc[w][gg][d] * f;
-      l += red_l[w][gg] * f;
-    }
-    float* dst = ws + (((size_t)b * n_heads + kvh * G + gg) * n_splits + split) * (D + 2);
-    dst[d] = a;
-    if (d == 0) {
-      dst[D] = mx;
-      dst[D + 1] = l;
-    }
-  }
-}
-
-template <int D>
-__global__ void attn_decode_combine_kernel(const float* __restrict__ ws, bf16_t* __restrict__ out, int n_splits);
-
-// =============================================================================== decode, fused
-// One kernel for a decode step's attention: rotate q and the new k (angles from the table),
-// store the new k, v in the cache and attend over the pages.  The new token's key and value
-// are taken from LDS where the loop reaches the token's own position, so no workgroup reads
-// what another one has just written.  With one split the result is written directly; with
-// more, the partial states go to the workspace and attn_decode_combine_kernel adds them.
-// (Combining inside this kernel by a ticket counter was tried: the device-scope fences it
-// needs write back and invalidate the L2 of every XCD and cost far more than the launch
-// they save.)
-template <int D, int G>
-__global__ __launch_bounds__(256) void attn_decode_fused_kernel(
-    const float* __restrict__ qkv, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int style,
-    bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out, const int32_t* __restrict__ tok_pos,
-    const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, float scale_log2, int window,
-    int n_splits, float* __restrict__ ws) {
-  constexpr int DL = D / 64;
-  constexpr int QC = D / 32;
   constexpr int HALF = D / 2;
   __shared__ float q_s[G][D];
   __shared__ float knew_s[D], vnew_s[D];
@@ -436,39 +304,45 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   const int pos = tok_pos[b];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int first_page = lo / RB_PAGE, last_page = pos / RB_PAGE;
-  const int row_width = (n_heads + 2 * n_kv) * D;
-  const float* src = qkv + (size_t)b * row_width;
-  const float* cr = cos_t ? cos_t + (size_t)pos * HALF : nullptr;
-  const float* sr = cos_t ? sin_t + (size_t)pos * HALF : nullptr;
+  const int32_t* pages = block_table + (size_t)b * bt_stride;
 
-  // ---- rotate the group's q heads and the kv head's new k; round through bfloat16 as the
-  // separate kernels do, so that both ways give the same numbers
-  for (int idx = tid; idx < (G + 1) * HALF; idx += 256) {
-    const int gg = idx / HALF, i = idx - gg * HALF;
-    const int i0 = style == 0 ? 2 * i : i, i1 = style == 0 ? 2 * i + 1 : i + HALF;
-    const float* h = gg < G ? src + (size_t)(kvh * G + gg) * D : src + (size_t)(n_heads + kvh) * D;
-    const float x0 = h[i0], x1 = h[i1];
-    float y0 = x0, y1 = x1;
-    if (cr) {
-      const float c = cr[i], sn = sr[i];
-      y0 = x0 * c - x1 * sn;
-      y1 = x0 * sn + x1 * c;
+  if (FUSED) {
+    const int row_width = (n_heads + 2 * n_kv) * D;
+    const float* src = qkv + (size_t)b * row_width;
+    const float* cr = cos_t ? cos_t + (size_t)pos * HALF : nullptr;
+    const float* sr = cos_t ? sin_t + (size_t)pos * HALF : nullptr;
+    for (int idx = tid; idx < (G + 1) * HALF; idx += 256) {
+      const int gg = idx / HALF, i = idx - gg * HALF;
+      const int i0 = style == 0 ? 2 * i : i, i1 = style == 0 ? 2 * i + 1 : i + HALF;
+      const float* h = gg < G ? src + (size_t)(kvh * G + gg) * D : src + (size_t)(n_heads + kvh) * D;
+      const float x0 = h[i0], x1 = h[i1];
+      float y0 = x0, y1 = x1;
+      if (cr) {
+        const float c = cr[i], sn = sr[i];
+        y0 = x0 * c - x1 * sn;
+        y1 = x0 * sn + x1 * c;
+      }
+      y0 = bf16_to_f32(f32_to_bf16(y0));
+      y1 = bf16_to_f32(f32_to_bf16(y1));
+      if (gg < G) {
+        q_s[gg][i0] = y0 * scale_log2;
+        q_s[gg][i1] = y1 * scale_log2;
+      } else {
+        knew_s[i0] = y0;
+        knew_s[i1] = y1;
+      }
     }
-    y0 = bf16_to_f32(f32_to_bf16(y0));
-    y1 = bf16_to_f32(f32_to_bf16(y1));
-    if (gg < G) {
-      q_s[gg][i0] = y0 * scale_log2;
-      q_s[gg][i1] = y1 * scale_log2;
-    } else {
-      knew_s[i0] = y0;
-      knew_s[i1] = y1;
+    for (int d = tid; d < D; d += 256)
+      vnew_s[d] = bf16_to_f32(f32_to_bf16(src[(size_t)(n_heads + n_kv + kvh) * D + d]));
+  } else {
+    for (int idx = tid; idx < G * D; idx += 256) {
+      const int gg = idx / D, d = idx % D;
+      q_s[gg][d] = bf16_to_f32(q_in[((size_t)b * n_heads + kvh * G + gg) * D + d]) * scale_log2;
     }
   }
-  for (int d = tid; d < D; d += 256)
-    vnew_s[d] = bf16_to_f32(f32_to_bf16(src[(size_t)(n_heads + n_kv + kvh) * D + d]));
   __syncthreads();
-  if (split == (last_page - first_page) % n_splits) {      // the workgroup that owns the last page stores them
-    const int page = block_table[(size_t)b * bt_stride + last_page];
+  if (FUSED && split == (last_page - first_page) % n_splits) {      // this workgroup owns the last page
+    const int page = pages[last_page];
     const size_t at = ((size_t)page * n_kv + kvh) * RB_PAGE * D + (size_t)(pos % RB_PAGE) * D;
     for (int d = tid; d < D; d += 256) {
       k_pages[at + d] = f32_to_bf16(knew_s[d]);
@@ -485,78 +359,100 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     for (int e = 0; e < DL; ++e) acc[gg][e] = 0.f;
   }
   const int j = lane >> 2, part = lane & 3;
-  for (int pg = first_page + split; pg <= last_page; pg += n_splits) {
-    const int page = block_table[(size_t)b * bt_stride + pg];
+  // this wave's pages: first_page + split + n_splits * (wave + 4 i)
+  for (int pg = first_page + split + n_splits * wave; pg <= last_page; pg += 4 * n_splits) {
+    const int page = pages[pg];
     const size_t base = ((size_t)page * n_kv + kvh) * RB_PAGE * D;
-    const int key0 = pg * RB_PAGE + wave * 16;
-    const int key = key0 + j;
-    const bool valid = key >= lo && key <= pos;
-    const bool is_new = key == pos;
-    float s[G];
+    // ---- all of the page's loads first: K quarter rows for 4 passes of 16 keys, V columns of 64 keys
+    uint4 kreg[4][QC];
+    uint32_t vreg[4][16];
 #pragma unroll
-    for (int gg = 0; gg < G; ++gg) s[gg] = 0.f;
-    const bf16_t* krow = k_pages + base + (size_t)(wave * 16 + j) * D + part * (D / 4);
+    for (int ps = 0; ps < 4; ++ps) {
+      const bf16_t* krow = k_pages + base + (size_t)(ps * 16 + j) * D + part * (D / 4);
 #pragma unroll
-    for (int cidx = 0; cidx < QC; ++cidx) {
-      const uint4 u = load16(krow + cidx * 8);
-      const uint32_t wds[4] = {u.x, u.y, u.z, u.w};
+      for (int cidx = 0; cidx < QC; ++cidx) kreg[ps][cidx] = load16(krow + cidx * 8);
+    }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int d = part * (D / 4) + cidx * 8 + 2 * e;
-        const float k0 = is_new ? knew_s[d] : bf16_bits_to_f32(wds[e] & 0xffffu);
-        const float k1 = is_new ? knew_s[d + 1] : bf16_bits_to_f32(wds[e] >> 16);
+    for (int ps = 0; ps < 4; ++ps) {
+      const bf16_t* vcol = v_pages + base + (size_t)(ps * 16) * D + lane * DL;
 #pragma unroll
-        for (int gg = 0; gg < G; ++gg) s[gg] = fmaf(k1, q_s[gg][d + 1], fmaf(k0, q_s[gg][d], s[gg]));
+      for (int jj = 0; jj < 16; ++jj) {
+        if (DL == 2)
+          vreg[ps][jj] = *reinterpret_cast<const uint32_t*>(vcol + (size_t)jj * D);
+        else
+          vreg[ps][jj] = (uint32_t)vcol[(size_t)jj * D].bits;
       }
     }
 #pragma unroll
-    for (int gg = 0; gg < G; ++gg) {
-      float v = s[gg];
-      v += __shfl_xor(v, 1, 64);
-      v += __shfl_xor(v, 2, 64);
-      if (!valid) v = -INFINITY;
-      float mx = v;
+    for (int ps = 0; ps < 4; ++ps) {
+      const int key0 = pg * RB_PAGE + ps * 16;
+      if (key0 > pos || key0 + 15 < lo) continue;          // nothing valid in this pass (uniform)
+      const int key = key0 + j;
+      const bool valid = key >= lo && key <= pos;
+      const bool is_new = FUSED && key == pos;
+      float s[G];
 #pragma unroll
-      for (int o = 4; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-      const float m_new = fmaxf(m_run[gg], mx);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float corr = exp2f(m_run[gg] - m_safe);
-      const float p = exp2f(v - m_safe);
-      float ps = p;
+      for (int gg = 0; gg < G; ++gg) s[gg] = 0.f;
 #pragma unroll
-      for (int o = 4; o < 64; o <<= 1) ps += __shfl_xor(ps, o, 64);
-      l_run[gg] = l_run[gg] * corr + ps;
-      m_run[gg] = m_new;
+      for (int cidx = 0; cidx < QC; ++cidx) {
+        const uint4 u = kreg[ps][cidx];
+        const uint32_t wds[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
-      for (int e = 0; e < DL; ++e) acc[gg][e] *= corr;
-      if (part == 0) p_s[wave][gg][j] = p;
-    }
-    __syncthreads();
-    int jj_lo = lo - key0;
-    if (jj_lo < 0) jj_lo = 0;
-    int jj_hi = pos - key0;
-    if (jj_hi > 15) jj_hi = 15;
-    const bf16_t* vcol = v_pages + base + (size_t)(wave * 16) * D + lane * DL;
-    for (int jj = jj_lo; jj <= jj_hi; ++jj) {
-      float v[DL];
-      if (key0 + jj == pos) {
+        for (int e = 0; e < 4; ++e) {
+          const int d = part * (D / 4) + cidx * 8 + 2 * e;
+          const float k0 = is_new ? knew_s[d] : bf16_bits_to_f32(wds[e] & 0xffffu);
+          const float k1 = is_new ? knew_s[d + 1] : bf16_bits_to_f32(wds[e] >> 16);
 #pragma unroll
-        for (int e = 0; e < DL; ++e) v[e] = vnew_s[lane * DL + e];
-      } else if (DL == 2) {
-        const uint32_t u = *reinterpret_cast<const uint32_t*>(vcol + (size_t)jj * D);
-        v[0] = bf16_bits_to_f32(u & 0xffffu);
-        v[DL - 1] = bf16_bits_to_f32(u >> 16);
-      } else {
-        v[0] = bf16_to_f32(vcol[(size_t)jj * D]);
+          for (int gg = 0; gg < G; ++gg) s[gg] = fmaf(k1, q_s[gg][d + 1], fmaf(k0, q_s[gg][d], s[gg]));
+        }
       }
 #pragma unroll
       for (int gg = 0; gg < G; ++gg) {
-        const float p = p_s[wave][gg][jj];
+        float v = s[gg];
+        v += __shfl_xor(v, 1, 64);
+        v += __shfl_xor(v, 2, 64);
+        if (!valid) v = -INFINITY;
+        float mx = v;
 #pragma unroll
-        for (int e = 0; e < DL; ++e) acc[gg][e] = fmaf(p, v[e], acc[gg][e]);
+        for (int o = 4; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        const float m_new = fmaxf(m_run[gg], mx);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = exp2f(m_run[gg] - m_safe);
+        const float p = exp2f(v - m_safe);
+        float psum = p;
+#pragma unroll
+        for (int o = 4; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
+        l_run[gg] = l_run[gg] * corr + psum;
+        m_run[gg] = m_new;
+#pragma unroll
+        for (int e = 0; e < DL; ++e) acc[gg][e] *= corr;
+        if (part == 0) p_s[wave][gg][j] = p;
       }
+      __builtin_amdgcn_wave_barrier();          // p_s is exchanged inside the wave only
+      // ---- weighted sum of the values; rows outside [lo, pos] may hold anything and are skipped
+#pragma unroll
+      for (int jj = 0; jj < 16; ++jj) {
+        const int kk = key0 + jj;
+        if (kk < lo || kk > pos) continue;
+        float v[DL];
+        if (FUSED && kk == pos) {
+#pragma unroll
+          for (int e = 0; e < DL; ++e) v[e] = vnew_s[lane * DL + e];
+        } else if (DL == 2) {
+          v[0] = bf16_bits_to_f32(vreg[ps][jj] & 0xffffu);
+          v[DL - 1] = bf16_bits_to_f32(vreg[ps][jj] >> 16);
+        } else {
+          v[0] = bf16_bits_to_f32(vreg[ps][jj]);
+        }
+#pragma unroll
+        for (int gg = 0; gg < G; ++gg) {
+          const float p = p_s[wave][gg][jj];
+#pragma unroll
+          for (int e = 0; e < DL; ++e) acc[gg][e] = fmaf(p, v[e], acc[gg][e]);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
     }
-    __syncthreads();
   }
 
   // ---- the four waves' states into one
@@ -596,58 +492,6 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   }
 }
 
-template <int D, int G>
-static void launch_decode_fused(const float* qkv, const float* cos_t, const float* sin_t, int style, bf16_t* k,
-                                bf16_t* v, bf16_t* out, const int32_t* tok_pos, const int32_t* bt, int bt_stride,
-                                int n_seqs, int n_heads, int n_kv, float sl2, int window, int n_splits, float* ws,
-                                hipStream_t s) {
-  dim3 grid(n_splits, n_kv, n_seqs);
-  attn_decode_fused_kernel<D, G><<<grid, 256, 0, s>>>(qkv, cos_t, sin_t, style, k, v, out, tok_pos, bt, bt_stride,
-                                                      n_heads, n_kv, sl2, window, n_splits, ws);
-  if (n_splits > 1) attn_decode_combine_kernel<D><<<n_seqs * n_heads, D, 0, s>>>(ws, out, n_splits);
-}
-
-extern "C" int rb_attention_decode_fused_bf16(const float* qkv, const float* cos, const float* sin, int style,
-                                              void* k_pages, void* v_pages, void* out, const int32_t* tok_pos,
-                                              const int32_t* block_table, int bt_stride, int n_seqs, int n_heads,
-                                              int n_kv_heads, int head_dim, float scale, int window, int n_splits,
-                                              float* workspace, void* stream) {
-  RB_REQUIRE(n_seqs > 0, "rb_attention_decode_fused_bf16: empty batch");
-  RB_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
-             "rb_attention_decode_fused_bf16: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
-  RB_REQUIRE(head_dim == 64 || head_dim == 128,
-             "rb_attention_decode_fused_bf16: head_dim %d not supported (64 or 128)", head_dim);
-  RB_REQUIRE(n_splits >= 1 && n_splits <= 65535, "rb_attention_decode_fused_bf16: bad split count %d", n_splits);
-  RB_REQUIRE(n_kv_heads <= 65535 && n_seqs <= 65535, "rb_attention_decode_fused_bf16: batch or head count too large");
-  RB_REQUIRE(window >= 0, "rb_attention_decode_fused_bf16: negative window");
-  RB_REQUIRE((cos == nullptr) == (sin == nullptr), "rb_attention_decode_fused_bf16: cos and sin tables go together");
-  RB_REQUIRE(style == 0 || style == 1, "rb_attention_decode_fused_bf16: unknown pairing style %d", style);
-  RB_REQUIRE(n_splits == 1 || workspace != nullptr, "rb_attention_decode_fused_bf16: splits need a workspace");
-  const int group = n_heads / n_kv_heads;
-  RB_REQUIRE(group == 1 || group == 2 || group == 4 || group == 8,
-             "rb_attention_decode_fused_bf16: %d query heads per kv head not supported (1, 2, 4, 8)", group);
-  hipStream_t s = (hipStream_t)stream;
-  const float sl2 = scale * LOG2E;
-#define RB_DECF(DV, GV)                                                                                          \
-  launch_decode_fused<DV, GV>(qkv, cos, sin, style, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out, tok_pos,    \
-                              block_table, bt_stride, n_seqs, n_heads, n_kv_heads, sl2, window, n_splits, workspace, \
-                              s)
-  if (head_dim == 128) {
-    if (group == 1) RB_DECF(128, 1);
-    else if (group == 2) RB_DECF(128, 2);
-    else if (group == 4) RB_DECF(128, 4);
-    else RB_DECF(128, 8);
-  } else {
-    if (group == 1) RB_DECF(64, 1);
-    else if (group == 2) RB_DECF(64, 2);
-    else if (group == 4) RB_DECF(64, 4);
-    else RB_DECF(64, 8);
-  }
-#undef RB_DECF
-  RB_LAUNCH_CHECK();
-  return 0;
-}
-
 template <int D>
 __global__ void attn_decode_combine_kernel(const float* __restrict__ ws, bf16_t* __restrict__ out, int n_splits) {
   const size_t row = blockIdx.x;            // sequence * heads + head
@@ -665,53 +509,80 @@ __global__ void attn_decode_combine_kernel(const float* __restrict__ ws, bf16_t*
   out[row * D + d] = f32_to_bf16(l > 0.f ? a / l : 0.f);
 }
 
-template <int D, int G>
-static void launch_decode(const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* out, const int32_t* tok_pos,
-                          const int32_t* bt, int bt_stride, int n_seqs, int n_heads, int n_kv, float sl2, int window,
-                          int n_splits, float* ws, hipStream_t s) {
-  dim3 grid(n_splits, n_kv, n_seqs);
-  attn_decode_kernel<D, G><<<grid, 256, 0, s>>>(q, k, v, tok_pos, bt, bt_stride, n_heads, n_kv, sl2, window,
-                                                n_splits, ws);
-  attn_decode_combine_kernel<D><<<n_seqs * n_heads, D, 0, s>>>(ws, out, n_splits);
+struct DecodeArgs {
+  const float* qkv;
+  const bf16_t* q;
+  const float* cos_t;
+  const float* sin_t;
+  int style;
+  bf16_t* k;
+  bf16_t* v;
+  bf16_t* out;
+  const int32_t* tok_pos;
+  const int32_t* bt;
+  int bt_stride, n_seqs, n_heads, n_kv;
+  float sl2;
+  int window, n_splits;
+  float* ws;
+};
+
+template <int D, int G, bool FUSED>
+static void launch_decode(const DecodeArgs& a, hipStream_t s) {
+  dim3 grid(a.n_splits, a.n_kv, a.n_seqs);
+  attn_decode_kernel<D, G, FUSED><<<grid, 256, 0, s>>>(a.qkv, a.q, a.cos_t, a.sin_t, a.style, a.k, a.v, a.out,
+                                                       a.tok_pos, a.bt, a.bt_stride, a.n_heads, a.n_kv, a.sl2,
+                                                       a.window, a.n_splits, a.ws);
+  if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits);
+}
+
+template <bool FUSED>
+static int dispatch_decode(const DecodeArgs& a, int head_dim, hipStream_t s, const char* who) {
+  RB_REQUIRE(a.n_seqs > 0, "%s: empty batch", who);
+  RB_REQUIRE(a.n_heads > 0 && a.n_kv > 0 && a.n_heads % a.n_kv == 0, "%s: bad head counts Hq=%d Hk=%d", who,
+             a.n_heads, a.n_kv);
+  RB_REQUIRE(head_dim == 64 || head_dim == 128, "%s: head_dim %d not supported (64 or 128; use rb_attention_generic)",
+             who, head_dim);
+  RB_REQUIRE(a.n_splits >= 1 && a.n_splits <= 65535, "%s: bad split count %d", who, a.n_splits);
+  RB_REQUIRE(a.n_kv <= 65535 && a.n_seqs <= 65535, "%s: batch or head count too large", who);
+  RB_REQUIRE(a.window >= 0, "%s: negative window", who);
+  RB_REQUIRE(a.n_splits == 1 || a.ws != nullptr, "%s: splits need a workspace", who);
+  const int group = a.n_heads / a.n_kv;
+  RB_REQUIRE(group == 1 || group == 2 || group == 4 || group == 8,
+             "%s: %d query heads per kv head not supported (1, 2, 4, 8; use rb_attention_generic)", who, group);
+  if (head_dim == 128) {
+    if (group == 1) launch_decode<128, 1, FUSED>(a, s);
+    else if (group == 2) launch_decode<128, 2, FUSED>(a, s);
+    else if (group == 4) launch_decode<128, 4, FUSED>(a, s);
+    else launch_decode<128, 8, FUSED>(a, s);
+  } else {
+    if (group == 1) launch_decode<64, 1, FUSED>(a, s);
+    else if (group == 2) launch_decode<64, 2, FUSED>(a, s);
+    else if (group == 4) launch_decode<64, 4, FUSED>(a, s);
+    else launch_decode<64, 8, FUSED>(a, s);
+  }
+  RB_LAUNCH_CHECK();
+  return 0;
 }
 
 extern "C" int rb_attention_decode_bf16(const void* q, const void* k_pages, const void* v_pages, void* out,
                                         const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
                                         int n_seqs, int n_heads, int n_kv_heads, int head_dim, float scale,
                                         int window, int n_splits, float* workspace, void* stream) {
-  RB_REQUIRE(n_seqs > 0, "rb_attention_decode_bf16: empty batch");
-  RB_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
-             "rb_attention_decode_bf16: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
-  RB_REQUIRE(head_dim == 64 || head_dim == 128,
-             "rb_attention_decode_bf16: head_dim %d not supported (64 or 128; use rb_attention_generic)", head_dim);
-  RB_REQUIRE(n_splits >= 1 && n_splits <= 65535, "rb_attention_decode_bf16: bad split count %d", n_splits);
-  RB_REQUIRE(n_kv_heads <= 65535 && n_seqs <= 65535, "rb_attention_decode_bf16: batch or head count too large");
-  RB_REQUIRE(window >= 0, "rb_attention_decode_bf16: negative window");
-  const int group = n_heads / n_kv_heads;
-  RB_REQUIRE(group == 1 || group == 2 || group == 4 || group == 8,
-             "rb_attention_decode_bf16: %d query heads per kv head not supported (1, 2, 4, 8; use "
-             "rb_attention_generic)", group);
-  hipStream_t s = (hipStream_t)stream;
-  const float sl2 = scale * LOG2E;
-  const bf16_t* qq = (const bf16_t*)q;
-  const bf16_t* kk = (const bf16_t*)k_pages;
-  const bf16_t* vv = (const bf16_t*)v_pages;
-  bf16_t* oo = (bf16_t*)out;
-#define RB_DEC(DV, GV)                                                                                         \
-  launch_decode<DV, GV>(qq, kk, vv, oo, tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, sl2, window, \
-                        n_splits, workspace, s)
-  if (head_dim == 128) {
-    if (group == 1) RB_DEC(128, 1);
-    else if (group == 2) RB_DEC(128, 2);
-    else if (group == 4) RB_DEC(128, 4);
-    else RB_DEC(128, 8);
-  } else {
-    if (group == 1) RB_DEC(64, 1);
-    else if (group == 2) RB_DEC(64, 2);
-    else if (group == 4) RB_DEC(64, 4);
-    else RB_DEC(64, 8);
-  }
-#undef RB_DEC
-  RB_LAUNCH_CHECK();
-  return 0;
+  DecodeArgs a = {nullptr, (const bf16_t*)q, nullptr, nullptr, 0, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out,
+                  tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, scale * LOG2E, window, n_splits,
+                  workspace};
+  return dispatch_decode<false>(a, head_dim, (hipStream_t)stream, "rb_attention_decode_bf16");
+}
+
+extern "C" int rb_attention_decode_fused_bf16(const float* qkv, const float* cos, const float* sin, int style,
+                                              void* k_pages, void* v_pages, void* out, const int32_t* tok_pos,
+                                              const int32_t* block_table, int bt_stride, int n_seqs, int n_heads,
+                                              int n_kv_heads, int head_dim, float scale, int window, int n_splits,
+                                              float* workspace, void* stream) {
+  RB_REQUIRE((cos == nullptr) == (sin == nullptr), "rb_attention_decode_fused_bf16: cos and sin tables go together");
+  RB_REQUIRE(style == 0 || style == 1, "rb_attention_decode_fused_bf16: unknown pairing style %d", style);
+  DecodeArgs a = {qkv, nullptr, cos, sin, style, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out,
+                  tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, scale * LOG2E, window, n_splits,
+                  workspace};
+  return dispatch_decode<true>(a, head_dim, (hipStream_t)stream, "rb_attention_decode_fused_bf16");
 }

@@ -70,12 +70,14 @@ class Kernels:
             "rb_attention_decode_bf16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
             "rb_attention_decode_fused_bf16": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
                                                _P, _P],
-            "rb_sample": [_P, _I, _I, _P, _P, _P, _P],
+            "rb_sample": [_P, _I, _I, _P, _P, _P, _P, _P],
         }
         for name, args in sig.items():
             fn = getattr(L, name)
             fn.argtypes = args
             fn.restype = _I
+        L.rb_sample_workspace_bytes.argtypes = [_I, _I]
+        L.rb_sample_workspace_bytes.restype = _I
         self.page_size = int(L.rb_page_size())
 
     # ------------------------------------------------------------------ helpers
@@ -241,15 +243,21 @@ class Kernels:
             int(n_splits), _ptr(workspace), self._stream()))
 
     def sample(self, logits: torch.Tensor, temperature: Optional[torch.Tensor], u: Optional[torch.Tensor],
-               tokens: torch.Tensor) -> None:
+               tokens: torch.Tensor, workspace: Optional[torch.Tensor] = None) -> None:
         n, vocab = logits.shape
         _check(logits, "logits", torch.float32)
         if temperature is not None:
             _check(temperature, "temperature", torch.float32, (n,))
             _check(u, "u", torch.float32, (n,))
         _check(tokens, "tokens", torch.int32, (n,))
+        need = int(self._lib.rb_sample_workspace_bytes(n, vocab))
+        if workspace is None:
+            workspace = torch.empty((need + 7) // 8, dtype=torch.int64, device=logits.device)
+        _check(workspace, "workspace", torch.int64)
+        if workspace.numel() * 8 < need:
+            raise KernelError("sampling workspace too small")
         self._ok(self._lib.rb_sample(_ptr(logits), n, vocab, _ptr(temperature), _ptr(u), _ptr(tokens),
-                                     self._stream()))
+                                     _ptr(workspace), self._stream()))
 
 
 _lock = threading.Lock()

@@ -13,6 +13,17 @@ import numpy as np
 import torch
 
 
+def decode_splits(n_seqs: int, n_kv_heads: int) -> int:
+    """Into how many workgroups the pages of one (sequence, kv head) are dealt in decode
+    attention: enough to give every compute unit about one workgroup, no more (each
+    workgroup already walks four pages at a time, and every split adds to the combination)."""
+    import os
+    forced = os.environ.get("RBITNET_DECODE_SPLITS")
+    if forced:
+        return max(1, int(forced))
+    return max(1, min(16, 256 // max(1, n_seqs * max(1, n_kv_heads))))
+
+
 class StepContext:
     def __init__(self, device, slots: Sequence[int], past_lens: Sequence[int], tokens: Sequence[Sequence[int]],
                  rows: Sequence[int], block_tables: Dict[int, List[List[int]]], n_kv_heads_hint: int = 1):
@@ -70,7 +81,7 @@ class StepContext:
         GPU, whatever the context length (each split strides over the pages)."""
         key = (n_heads, head_dim, n_kv_heads)
         if key not in self._workspaces:
-            n_splits = max(1, min(32, 2048 // max(1, self.n_seqs * n_heads)))
+            n_splits = decode_splits(self.n_seqs, n_kv_heads)
             ws = torch.empty(self.n_seqs * n_heads * n_splits * (head_dim + 2), dtype=torch.float32,
                              device=self.device)
             self._workspaces[key] = (n_splits, ws)

@@ -18,6 +18,7 @@ import numpy as np
 import torch
 
 from ..cache.pages import pages_for
+from .context import decode_splits
 
 
 class _StaticContext:
@@ -74,7 +75,7 @@ class _StaticContext:
     def decode_workspace(self, n_heads: int, head_dim: int, n_kv_heads: int = 1):
         key = (n_heads, head_dim, n_kv_heads)
         if key not in self._workspaces:
-            n_splits = max(1, min(32, 2048 // max(1, self.n_seqs * n_heads)))
+            n_splits = decode_splits(self.n_seqs, n_kv_heads)
             ws = torch.empty(self.n_seqs * n_heads * n_splits * (head_dim + 2), dtype=torch.float32,
                              device=self.device)
             self._workspaces[key] = (n_splits, ws)

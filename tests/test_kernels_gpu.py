@@ -95,7 +95,7 @@ def test_embed_gather(lib, dtype):
     assert torch.equal(out.cpu(), table.float()[ids.long()])
 
 
-@pytest.mark.parametrize("width,eps", [(50, 1e-5), (1000, 1e-6), (4100, 1e-2)])
+@pytest.mark.parametrize("width,eps", [(50, 1e-5), (1000, 1e-6), (4100, 1e-2), (4096, 1e-5), (12000, 1e-5)])
 def test_add_rmsnorm(lib, width, eps):
     g = torch.Generator().manual_seed(width)
     x = torch.randn(6, width, generator=g) * 1e-2        # small, so that eps matters
@@ -306,8 +306,8 @@ def test_far_key_stands_out(lib):
 def test_sample_greedy_and_inverse_cdf(lib):
     from plain_llama import sample_token
     g = torch.Generator().manual_seed(11)
-    logits = torch.randn(7, 1000, generator=g) * 3
-    logits[2, 5] = logits[2, 900] = 50.0                 # equal maxima: the lowest index wins
+    logits = torch.randn(7, 9001, generator=g) * 3        # three chunks, the last one short
+    logits[2, 5] = logits[2, 8900] = 50.0                # equal maxima: the lowest index wins
     logits[3, 17] = float("nan")
     tokens = torch.empty(7, dtype=torch.int32, device=DEV)
     lib.sample(logits.to(DEV), None, None, tokens)
@@ -316,6 +316,7 @@ def test_sample_greedy_and_inverse_cdf(lib):
     assert tokens.tolist() == want
     temps = torch.tensor([0.8, 0.0, 1.5, 0.3, 1.0, 0.8, 2.0])
     us = torch.tensor([0.0, 0.5, 0.999999, 0.25, 0.5, 0.73, 0.1])
+    logits[4, 4096:8192] += 6.0                          # most of the mass in the middle chunk
     lib.sample(logits.to(DEV), temps.to(DEV), us.to(DEV), tokens)
     for r in range(7):
         row = torch.nan_to_num(logits[r], nan=-float("inf"))
