@@ -285,6 +285,51 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
 // workspace and attn_decode_combine_kernel adds them.  (Combining inside this kernel by a
 // ticket counter was tried: the device-scope fences it needs write back and invalidate the
 // L2 of every XCD and cost far more than the launch they save.)
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+  union {
+    uint32_t u;
+    bf16x2_t v;
+  } x, y;
+  x.u = a;
+  y.u = b;
+  return __builtin_amdgcn_fdot2_f32_bf16(x.v, y.v, c, false);
+}
+// Cross-lane moves without LDS traffic (data-parallel primitives of the vector unit).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// sum over the 4 lanes of a quad; every lane gets it
+__device__ __forceinline__ float quad_sum(float v) {
+  v += dpp_move<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  return v;
+}
+// Reductions over the 16 quads of a wave for values that are equal within each quad: rotate
+// the rows of 16 lanes by 4 and 8, then combine the four rows through scalar registers.
+__device__ __forceinline__ float quads_max(float v) {
+  v = fmaxf(v, dpp_move<0x124>(v));      // row_ror:4
+  v = fmaxf(v, dpp_move<0x128>(v));      // row_ror:8
+  const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+__device__ __forceinline__ float quads_sum(float v) {
+  v += dpp_move<0x124>(v);
+  v += dpp_move<0x128>(v);
+  const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return (r0 + r1) + (r2 + r3);
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {      // lane is the same for the whole wave
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
 template <int D, int G, bool FUSED>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const float* __restrict__ qkv, const bf16_t* __restrict__ q_in, const float* __restrict__ cos_t,
@@ -293,10 +338,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws) {
   constexpr int DL = D / 64;          // output elements per lane
   constexpr int QC = D / 32;          // 16-byte chunks of a quarter row of K
+  constexpr int QP = D / 8;           // bfloat16 pairs of a quarter row
   constexpr int HALF = D / 2;
-  __shared__ float q_s[G][D];
-  __shared__ float knew_s[D], vnew_s[D];
-  __shared__ float p_s[4][G][16];
+  __shared__ __attribute__((aligned(16))) uint16_t q_h[G][D];
+  __shared__ __attribute__((aligned(16))) uint16_t knew_h[D], vnew_h[D];
   __shared__ float red_m[4][G], red_l[4][G];
   __shared__ float red_acc[4][G][D];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -305,7 +350,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int first_page = lo / RB_PAGE, last_page = pos / RB_PAGE;
   const int32_t* pages = block_table + (size_t)b * bt_stride;
+  const int j = lane >> 2, part = lane & 3;
 
+  const int pg_first = first_page + split + n_splits * wave;
+
+  // ---- q of the G heads as packed bfloat16 pairs in registers: this lane's quarter of each row
+  uint32_t q_pk[G][QP];
   if (FUSED) {
     const int row_width = (n_heads + 2 * n_kv) * D;
     const float* src = qkv + (size_t)b * row_width;
@@ -322,31 +372,36 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         y0 = x0 * c - x1 * sn;
         y1 = x0 * sn + x1 * c;
       }
-      y0 = bf16_to_f32(f32_to_bf16(y0));
-      y1 = bf16_to_f32(f32_to_bf16(y1));
-      if (gg < G) {
-        q_s[gg][i0] = y0 * scale_log2;
-        q_s[gg][i1] = y1 * scale_log2;
-      } else {
-        knew_s[i0] = y0;
-        knew_s[i1] = y1;
+      uint16_t* dst = gg < G ? q_h[gg] : knew_h;
+      dst[i0] = f32_to_bf16_bits(y0);
+      dst[i1] = f32_to_bf16_bits(y1);
+    }
+    for (int d = tid; d < D; d += 256) vnew_h[d] = f32_to_bf16_bits(src[(size_t)(n_heads + n_kv + kvh) * D + d]);
+    __syncthreads();
+#pragma unroll
+    for (int gg = 0; gg < G; ++gg)
+#pragma unroll
+      for (int i = 0; i < QP; ++i) q_pk[gg][i] = *reinterpret_cast<const uint32_t*>(&q_h[gg][part * (D / 4) + 2 * i]);
+    if (split == (last_page - first_page) % n_splits) {      // this workgroup owns the last page
+      const int page = pages[last_page];
+      const size_t at = ((size_t)page * n_kv + kvh) * RB_PAGE * D + (size_t)(pos % RB_PAGE) * D;
+      for (int d = tid; d < D; d += 256) {
+        k_pages[at + d].bits = knew_h[d];
+        v_pages[at + d].bits = vnew_h[d];
       }
     }
-    for (int d = tid; d < D; d += 256)
-      vnew_s[d] = bf16_to_f32(f32_to_bf16(src[(size_t)(n_heads + n_kv + kvh) * D + d]));
   } else {
-    for (int idx = tid; idx < G * D; idx += 256) {
-      const int gg = idx / D, d = idx % D;
-      q_s[gg][d] = bf16_to_f32(q_in[((size_t)b * n_heads + kvh * G + gg) * D + d]) * scale_log2;
-    }
-  }
-  __syncthreads();
-  if (FUSED && split == (last_page - first_page) % n_splits) {      // this workgroup owns the last page
-    const int page = pages[last_page];
-    const size_t at = ((size_t)page * n_kv + kvh) * RB_PAGE * D + (size_t)(pos % RB_PAGE) * D;
-    for (int d = tid; d < D; d += 256) {
-      k_pages[at + d] = f32_to_bf16(knew_s[d]);
-      v_pages[at + d] = f32_to_bf16(vnew_s[d]);
+#pragma unroll
+    for (int gg = 0; gg < G; ++gg) {
+      const bf16_t* qrow = q_in + ((size_t)b * n_heads + kvh * G + gg) * D + part * (D / 4);
+#pragma unroll
+      for (int c = 0; c < QC; ++c) {
+        const uint4 u = load16(qrow + c * 8);
+        q_pk[gg][4 * c + 0] = u.x;
+        q_pk[gg][4 * c + 1] = u.y;
+        q_pk[gg][4 * c + 2] = u.z;
+        q_pk[gg][4 * c + 3] = u.w;
+      }
     }
   }
 
@@ -358,12 +413,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 #pragma unroll
     for (int e = 0; e < DL; ++e) acc[gg][e] = 0.f;
   }
-  const int j = lane >> 2, part = lane & 3;
-  // this wave's pages: first_page + split + n_splits * (wave + 4 i)
-  for (int pg = first_page + split + n_splits * wave; pg <= last_page; pg += 4 * n_splits) {
+  // this wave's pages: first_page + split + n_splits * (wave + 4 i).  All of a page's loads
+  // are issued before the first is used.  (Requesting the next page's keys ahead was tried:
+  // the wave is bound by its arithmetic, not by the loads, and the extra registers cost a
+  // workgroup per compute unit.)
+  const int pg_step = 4 * n_splits;
+  auto work_page = [&](int pg) {
     const int page = pages[pg];
     const size_t base = ((size_t)page * n_kv + kvh) * RB_PAGE * D;
-    // ---- all of the page's loads first: K quarter rows for 4 passes of 16 keys, V columns of 64 keys
     uint4 kreg[4][QC];
     uint32_t vreg[4][16];
 #pragma unroll
@@ -386,74 +443,68 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 #pragma unroll
     for (int ps = 0; ps < 4; ++ps) {
       const int key0 = pg * RB_PAGE + ps * 16;
-      if (key0 > pos || key0 + 15 < lo) continue;          // nothing valid in this pass (uniform)
+      if (key0 > pos || key0 + 15 < lo) continue;          // nothing valid in this pass (same for the whole wave)
       const int key = key0 + j;
       const bool valid = key >= lo && key <= pos;
-      const bool is_new = FUSED && key == pos;
+      if (FUSED && pos >= key0 && pos < key0 + 16 && key == pos) {
+        // the token's own key is not in the cache yet (or only just): take it from LDS
+#pragma unroll
+        for (int cidx = 0; cidx < QC; ++cidx)
+          kreg[ps][cidx] = *reinterpret_cast<const uint4*>(&knew_h[part * (D / 4) + cidx * 8]);
+      }
       float s[G];
 #pragma unroll
       for (int gg = 0; gg < G; ++gg) s[gg] = 0.f;
 #pragma unroll
       for (int cidx = 0; cidx < QC; ++cidx) {
-        const uint4 u = kreg[ps][cidx];
-        const uint32_t wds[4] = {u.x, u.y, u.z, u.w};
+        const uint32_t wds[4] = {kreg[ps][cidx].x, kreg[ps][cidx].y, kreg[ps][cidx].z, kreg[ps][cidx].w};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int d = part * (D / 4) + cidx * 8 + 2 * e;
-          const float k0 = is_new ? knew_s[d] : bf16_bits_to_f32(wds[e] & 0xffffu);
-          const float k1 = is_new ? knew_s[d + 1] : bf16_bits_to_f32(wds[e] >> 16);
+        for (int e = 0; e < 4; ++e)
 #pragma unroll
-          for (int gg = 0; gg < G; ++gg) s[gg] = fmaf(k1, q_s[gg][d + 1], fmaf(k0, q_s[gg][d], s[gg]));
-        }
+          for (int gg = 0; gg < G; ++gg) s[gg] = dot2_bf16(wds[e], q_pk[gg][4 * cidx + e], s[gg]);
       }
+      float p[G];
 #pragma unroll
       for (int gg = 0; gg < G; ++gg) {
-        float v = s[gg];
-        v += __shfl_xor(v, 1, 64);
-        v += __shfl_xor(v, 2, 64);
-        if (!valid) v = -INFINITY;
-        float mx = v;
-#pragma unroll
-        for (int o = 4; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-        const float m_new = fmaxf(m_run[gg], mx);
+        float v = quad_sum(s[gg]);
+        v = valid ? v * scale_log2 : -INFINITY;
+        const float m_new = fmaxf(m_run[gg], quads_max(v));
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float corr = exp2f(m_run[gg] - m_safe);
-        const float p = exp2f(v - m_safe);
-        float psum = p;
-#pragma unroll
-        for (int o = 4; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
-        l_run[gg] = l_run[gg] * corr + psum;
+        const float corr = __builtin_amdgcn_exp2f(m_run[gg] - m_safe);
+        p[gg] = __builtin_amdgcn_exp2f(v - m_safe);
+        l_run[gg] = l_run[gg] * corr + quads_sum(p[gg]);
         m_run[gg] = m_new;
 #pragma unroll
         for (int e = 0; e < DL; ++e) acc[gg][e] *= corr;
-        if (part == 0) p_s[wave][gg][j] = p;
       }
-      __builtin_amdgcn_wave_barrier();          // p_s is exchanged inside the wave only
-      // ---- weighted sum of the values; rows outside [lo, pos] may hold anything and are skipped
+      // ---- weighted sum of the values: key jj's probability sits in lanes 4 jj .. 4 jj + 3;
+      // rows outside [lo, pos] may hold anything and are made zero
+      uint32_t vnew_pk = 0;
+      if (FUSED) {
+        if (DL == 2)
+          vnew_pk = *reinterpret_cast<const uint32_t*>(&vnew_h[lane * DL]);
+        else
+          vnew_pk = vnew_h[lane];
+      }
 #pragma unroll
       for (int jj = 0; jj < 16; ++jj) {
         const int kk = key0 + jj;
-        if (kk < lo || kk > pos) continue;
+        uint32_t raw = vreg[ps][jj];
+        if (FUSED && kk == pos) raw = vnew_pk;
+        if (kk < lo || kk > pos) raw = 0;
         float v[DL];
-        if (FUSED && kk == pos) {
-#pragma unroll
-          for (int e = 0; e < DL; ++e) v[e] = vnew_s[lane * DL + e];
-        } else if (DL == 2) {
-          v[0] = bf16_bits_to_f32(vreg[ps][jj] & 0xffffu);
-          v[DL - 1] = bf16_bits_to_f32(vreg[ps][jj] >> 16);
-        } else {
-          v[0] = bf16_bits_to_f32(vreg[ps][jj]);
-        }
+        v[0] = bf16_bits_to_f32(raw & 0xffffu);
+        if (DL == 2) v[DL - 1] = bf16_bits_to_f32(raw >> 16);
 #pragma unroll
         for (int gg = 0; gg < G; ++gg) {
-          const float p = p_s[wave][gg][jj];
+          const float pj = lane_value(p[gg], 4 * jj);
 #pragma unroll
-          for (int e = 0; e < DL; ++e) acc[gg][e] = fmaf(p, v[e], acc[gg][e]);
+          for (int e = 0; e < DL; ++e) acc[gg][e] = fmaf(pj, v[e], acc[gg][e]);
         }
       }
-      __builtin_amdgcn_wave_barrier();
     }
-  }
+  };
+  for (int pg = pg_first; pg <= last_page; pg += pg_step) work_page(pg);
 
   // ---- the four waves' states into one
 #pragma unroll
