@@ -7,9 +7,10 @@
 //    slice of K, streams them with 16-byte loads straight into MFMA operands, and the
 //    waves of a workgroup add their partial sums through LDS (no atomics: the sum order
 //    is fixed).
-//  * tiled (M > 64, prefill): 128 x 128 x 64 tiles through double-buffered LDS, 4 waves
-//    of 64 x 64, tile order arranged so that the workgroups an XCD runs together share
-//    their W and A tiles in that XCD's L2.
+//  * tiled (M > 64, prefill): 128 x 128, 256 x 128 or 256 x 256 tiles (depth 64) through
+//    double-buffered LDS, one wave per 64 x 64 or 128 x 64 piece, the next tile's global
+//    loads in flight in registers, tile order arranged so that the workgroups an XCD runs
+//    together share their W and A tiles in that XCD's L2.
 //
 // Epilogue 1 expects W with gate and up rows interleaved in blocks of 16 and writes
 // silu(gate) * up (llama/model.rs:297-302 of the reference) instead of the two products.
@@ -416,15 +417,16 @@ static bool try_resident(const bf16_t* x, const bf16_t* w, void* c, int m, int n
 #define TG_LD 72          // bf16 elements per LDS row: 64 + 8 of padding, so that the 16 lanes
                           // of a quarter wave read 16 different 16-byte bank groups
 
-template <int BN, int BM, int WN, int WM, int EPI, typename TO>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
+template <int BN, int BM, int WN, int WM, int P, int EPI, bool KTAIL, typename TO>
+__global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
                                                          const bf16_t* __restrict__ w, TO* __restrict__ c,
                                                          int m, int n, int k, int m_tiles, int n_tiles) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   constexpr int TN = WN / 32, TM = WM / 32;
   constexpr int WAVES_N = BN / WN;
-  constexpr int W_CHUNKS = BN * 8 / 256, X_CHUNKS = BM * 8 / 256;
-  static_assert((BN / WN) * (BM / WM) == 4, "four waves");
+  constexpr int NT = 64 * (BN / WN) * (BM / WM);      // threads: one wave per WN x WM piece of the tile
+  constexpr int W_CHUNKS = BN * 8 / NT, X_CHUNKS = BM * 8 / NT;
+  static_assert(BN * 8 % NT == 0 && BM * 8 % NT == 0 && NT % 8 == 0, "tile does not divide among the threads");
   bf16_t* ws = reinterpret_cast<bf16_t*>(smem);                      // [2][BN][TG_LD]
   bf16_t* xs = ws + 2 * BN * TG_LD;                                  // [2][BM][TG_LD]
 
@@ -453,59 +455,120 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  uint4 wreg[W_CHUNKS], xreg[X_CHUNKS];
-  auto load_global = [&](int k0) {
+  // ---- pipeline: tile kt is multiplied out of LDS while tiles kt + 1 .. kt + P - 1 are on
+  // their way from memory in registers (P - 1 tiles of latency hidden) and one of them is
+  // moved into the other LDS buffer.  Loads carry no conditions: rows beyond N or M are read
+  // from the last row and never stored, chunks beyond K are read from the last chunk and
+  // zeroed on their way into LDS.  (With conditions the compiler cannot count outstanding
+  // loads and waits for all of them.)
+  uint4 wreg[P][W_CHUNKS], xreg[P][X_CHUNKS];
+  // addresses: a 64-bit base per tile (the same for the whole workgroup) plus a 32-bit
+  // element offset per chunk; a tile spans at most 256 rows, so the offsets fit
+  const bf16_t* wtile = w + (size_t)n0 * k;
+  const bf16_t* xtile = x + (size_t)m0 * k;
+  uint32_t woff[W_CHUNKS], xoff[X_CHUNKS];
+#pragma unroll
+  for (int i = 0; i < W_CHUNKS; ++i) {
+    int row = (tid + NT * i) / 8;
+    if (n0 + row > n - 1) row = n - 1 - n0;
+    woff[i] = (uint32_t)row * (uint32_t)k;
+  }
+#pragma unroll
+  for (int i = 0; i < X_CHUNKS; ++i) {
+    int row = (tid + NT * i) / 8;
+    if (m0 + row > m - 1) row = m - 1 - m0;
+    xoff[i] = (uint32_t)row * (uint32_t)k;
+  }
+  const int kc = (tid % 8) * 8;             // this thread's chunk offset inside a tile (the same for all i)
+  auto load_global = [&](int slot, int kt) {
+    int col = kt * TG_BK + kc;
+    if (col > k - 8) col = k - 8;           // beyond K: any valid address; the data is zeroed in store_lds
+#pragma unroll
+    for (int i = 0; i < W_CHUNKS; ++i) wreg[slot][i] = load16(wtile + (woff[i] + (uint32_t)col));
+#pragma unroll
+    for (int i = 0; i < X_CHUNKS; ++i) xreg[slot][i] = load16(xtile + (xoff[i] + (uint32_t)col));
+  };
+  auto store_lds = [&](int slot, int kt) {
+    const int buf = kt & 1;
+    const bool in = !KTAIL || kt * TG_BK + kc < k;
 #pragma unroll
     for (int i = 0; i < W_CHUNKS; ++i) {
-      const int q = tid + 256 * i;
-      const int row = n0 + q / 8, kk = k0 + (q % 8) * 8;
-      wreg[i] = (row < n && kk < k) ? load16(w + (size_t)row * k + kk) : zero16();
+      const int q = tid + NT * i;
+      *reinterpret_cast<uint4*>(ws + ((size_t)buf * BN + q / 8) * TG_LD + kc) = in ? wreg[slot][i] : zero16();
     }
 #pragma unroll
     for (int i = 0; i < X_CHUNKS; ++i) {
-      const int q = tid + 256 * i;
-      const int row = m0 + q / 8, kk = k0 + (q % 8) * 8;
-      xreg[i] = (row < m && kk < k) ? load16(x + (size_t)row * k + kk) : zero16();
+      const int q = tid + NT * i;
+      *reinterpret_cast<uint4*>(xs + ((size_t)buf * BM + q / 8) * TG_LD + kc) = in ? xreg[slot][i] : zero16();
     }
   };
-  auto store_lds = [&](int buf) {
+  auto multiply = [&](int kt) {
+    const bf16_t* wb = ws + (size_t)(kt & 1) * BN * TG_LD;
+    const bf16_t* xb = xs + (size_t)(kt & 1) * BM * TG_LD;
+    if (NT <= 256) {
+      // fragments of k-step ks + 1 are requested from LDS before the MFMAs of k-step ks
+      Frag8 a[2][TN], b[2][TM];
+      auto load_frags = [&](int buf2, int ks) {
 #pragma unroll
-    for (int i = 0; i < W_CHUNKS; ++i) {
-      const int q = tid + 256 * i;
-      *reinterpret_cast<uint4*>(ws + ((size_t)buf * BN + q / 8) * TG_LD + (q % 8) * 8) = wreg[i];
-    }
+        for (int i = 0; i < TN; ++i)
+          a[buf2][i].u = *reinterpret_cast<const uint4*>(wb + (size_t)(wn0 + 32 * i + l32) * TG_LD + ks * 16 + g * 8);
 #pragma unroll
-    for (int i = 0; i < X_CHUNKS; ++i) {
-      const int q = tid + 256 * i;
-      *reinterpret_cast<uint4*>(xs + ((size_t)buf * BM + q / 8) * TG_LD + (q % 8) * 8) = xreg[i];
+        for (int j = 0; j < TM; ++j)
+          b[buf2][j].u = *reinterpret_cast<const uint4*>(xb + (size_t)(wm0 + 32 * j + l32) * TG_LD + ks * 16 + g * 8);
+      };
+      load_frags(0, 0);
+#pragma unroll
+      for (int ks = 0; ks < TG_BK / 16; ++ks) {
+        if (ks + 1 < TG_BK / 16) load_frags((ks + 1) & 1, ks + 1);
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+          for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[ks & 1][i], b[ks & 1][j], acc[i][j]);
+      }
+    } else {
+      // 8 waves: two per SIMD cover each other's LDS latency, and registers are scarce
+#pragma unroll
+      for (int ks = 0; ks < TG_BK / 16; ++ks) {
+        Frag8 a[TN], b[TM];
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+          a[i].u = *reinterpret_cast<const uint4*>(wb + (size_t)(wn0 + 32 * i + l32) * TG_LD + ks * 16 + g * 8);
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+          b[j].u = *reinterpret_cast<const uint4*>(xb + (size_t)(wm0 + 32 * j + l32) * TG_LD + ks * 16 + g * 8);
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+          for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+      }
     }
   };
 
   const int k_tiles = (k + TG_BK - 1) / TG_BK;
-  load_global(0);
-  store_lds(0);
+  // tiles beyond the last are loaded as well (clamped) and never stored: the loop body stays
+  // free of conditions on loads
+#pragma unroll
+  for (int sl = 0; sl < P; ++sl) load_global(sl, sl);
+  store_lds(0, 0);
   __syncthreads();
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < k_tiles) load_global((kt + 1) * TG_BK);
-    const bf16_t* wb = ws + (size_t)buf * BN * TG_LD;
-    const bf16_t* xb = xs + (size_t)buf * BM * TG_LD;
+  int kt = 0;
+  for (; kt + P <= k_tiles; kt += P) {        // P iterations per trip, so that the register slots are static
 #pragma unroll
-    for (int ks = 0; ks < TG_BK / 16; ++ks) {
-      Frag8 a[TN], b[TM];
-#pragma unroll
-      for (int i = 0; i < TN; ++i)
-        a[i].u = *reinterpret_cast<const uint4*>(wb + (size_t)(wn0 + 32 * i + l32) * TG_LD + ks * 16 + g * 8);
-#pragma unroll
-      for (int j = 0; j < TM; ++j)
-        b[j].u = *reinterpret_cast<const uint4*>(xb + (size_t)(wm0 + 32 * j + l32) * TG_LD + ks * 16 + g * 8);
-#pragma unroll
-      for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+    for (int u = 0; u < P; ++u) {
+      // slot u held tile kt + u (now in LDS): reuse it for tile kt + u + P
+      load_global(u, kt + u + P);
+      multiply(kt + u);
+      if (kt + u + 1 < k_tiles) store_lds((u + 1) % P, kt + u + 1);
+      __syncthreads();
     }
-    if (kt + 1 < k_tiles) store_lds(buf ^ 1);
-    __syncthreads();
+  }
+#pragma unroll
+  for (int u = 0; u < P; ++u) {               // the last k_tiles % P tiles
+    if (kt + u < k_tiles) {
+      multiply(kt + u);
+      if (kt + u + 1 < k_tiles) store_lds((u + 1) % P, kt + u + 1);
+      __syncthreads();
+    }
   }
 
   // ---- lane holds, per (i, j): token m0 + wm0 + 32 j + l32, W rows base + 8 (e / 4) + 4 g + e % 4
@@ -535,24 +598,50 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     }
 }
 
-template <int EPI, typename TO>
-static int launch_tiled(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
-  constexpr int BN = 128, BM = 128;
+static int g_tile_cfg = 0;
+extern "C" void rb_tune_tiles(int cfg) { g_tile_cfg = cfg; }      // experiments only; 0 = built-in choice
+
+template <int BN, int BM, int WN, int WM, int P, int EPI, typename TO>
+static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
   const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
   const long long tiles = (long long)m_tiles * n_tiles;
   RB_REQUIRE(tiles < (1LL << 30), "rb_gemm_bf16: too many tiles");
   const size_t lds = (size_t)2 * (BN + BM) * TG_LD * sizeof(bf16_t);
-  auto kern = gemm_tiled_kernel<BN, BM, 64, 64, EPI, TO>;
-  static bool configured = false;
-  if (!configured) {
+  const bool tail = k % TG_BK != 0;
+  auto kern = tail ? gemm_tiled_kernel<BN, BM, WN, WM, P, EPI, true, TO>
+                   : gemm_tiled_kernel<BN, BM, WN, WM, P, EPI, false, TO>;
+  static bool configured[2] = {false, false};
+  if (!configured[tail]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     RB_REQUIRE(e == hipSuccess, "rb_gemm_bf16: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    configured = true;
+    configured[tail] = true;
   }
   const int grid = (int)((tiles + 7) / 8 * 8);
-  kern<<<grid, 256, lds, s>>>(x, w, (TO*)c, m, n, k, m_tiles, n_tiles);
+  kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, m, n, k, m_tiles, n_tiles);
   return 0;
+}
+
+// Which tile for which product.  Measured on the Llama-3-8B products at M = 2048 and 8192:
+// the kernel is bound by what it pulls from L2 (a 128 x 128 tile needs 1 byte per 64 flop), so
+// the largest tile that still gives every compute unit work wins: 256 x 256 (8 waves) when
+// there are at least ~160 such tiles, 256 x 128 for long K with at least ~200 tiles, else
+// 128 x 128.
+template <int EPI, typename TO>
+static int launch_tiled(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
+  int cfg = g_tile_cfg;
+  if (cfg == 0) {
+    const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
+    const long long t256x128 = (long long)((m + 127) / 128) * ((n + 255) / 256);
+    if (t256 >= 160) cfg = 3;
+    else if (k >= 8192 && t256x128 >= 200) cfg = 2;
+    else cfg = 1;
+  }
+  switch (cfg) {
+    case 3: return launch_tiled_cfg<256, 256, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+    case 2: return launch_tiled_cfg<256, 128, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+    default: return launch_tiled_cfg<128, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+  }
 }
 
 static int g_use_resident = 1;
