@@ -23,8 +23,8 @@
 #define LOG2E 1.4426950408889634f
 
 // =============================================================================== prefill
-template <int D>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+template <int D, int NW>
+__global__ __launch_bounds__(64 * NW) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     bf16_t* __restrict__ out, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ past_len,
     const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, float scale_log2, int window,
@@ -32,7 +32,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   constexpr int KLD = D + 8;          // K tile row: D + 8 elements, rows 16 bytes apart in bank space
   constexpr int VLD = RB_PAGE + 8;    // V^T tile row: 64 keys + 8
   constexpr int DC = D / 8;           // 16-byte chunks per row
-  constexpr int KCH = RB_PAGE * DC / 256;
+  constexpr int NT = 64 * NW;
+  constexpr int KCH = RB_PAGE * DC / NT;
   __shared__ __attribute__((aligned(16))) bf16_t ks[RB_PAGE * KLD];
   __shared__ __attribute__((aligned(16))) bf16_t vt[D * VLD];
 
@@ -43,7 +44,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int groups_per_kv = group / gw;
   const int kvh = blockIdx.y / groups_per_kv;
   const int head = kvh * group + (blockIdx.y % groups_per_kv) * gw + (wave % gw);
-  const int q_per_wg = 32 * (4 / gw);
+  const int q_per_wg = 32 * (NW / gw);
   const int seq_start = cu_seqlens[b];
   const int q_len = cu_seqlens[b + 1] - seq_start;
   const int past = past_len[b];
@@ -73,11 +74,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int first_tile = wg_lo / RB_PAGE;
   const int last_tile = (past + wg_q_end) / RB_PAGE;
   int wave_first = first_tile, wave_last = -1;
+  int wave_min_pos = 0, wave_max_lo = 0;      // a tile all of whose keys lie in [wave_max_lo, wave_min_pos] needs no mask
   if (wave_on) {
     const int w_end = (q0 + 32 < q_len ? q0 + 32 : q_len) - 1;
     wave_last = (past + w_end) / RB_PAGE;
     const int w_min = past + q0;
     wave_first = ((window > 0 && w_min - window + 1 > 0) ? w_min - window + 1 : 0) / RB_PAGE;
+    wave_min_pos = w_min;
+    wave_max_lo = (window > 0 && past + w_end - window + 1 > 0) ? past + w_end - window + 1 : 0;
   }
 
   float m_run = -INFINITY, l_run = 0.f;
@@ -91,7 +95,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   // V: a thread takes 4 consecutive keys x 8 consecutive d (one 16-byte chunk of 4 rows)
   const int v_dchunk = (tid & 3) + 4 * (tid >> 6);
   const int v_quad = (tid >> 2) & 15;
-  const bool v_on = v_dchunk < DC;
+  const bool v_on = tid < 256 && v_dchunk < DC;
   // place of the quad in the permuted key order of a V^T row (see the second MFMA below)
   const int qq = v_quad & 7;
   const int v_col = (v_quad >> 3) * 32 + (2 * (qq >> 2) + (qq & 1)) * 8 + ((qq >> 1) & 1) * 4;
@@ -102,7 +106,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const size_t base = ((size_t)page * n_kv + kvh) * RB_PAGE * D;
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
-      const int c = tid + 256 * i;
+      const int c = tid + NT * i;
       kreg[i] = load16(k_pages + base + (size_t)(c / DC) * D + (c % DC) * 8);
     }
     if (v_on) {
@@ -118,7 +122,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   auto store_tile = [&]() {
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
-      const int c = tid + 256 * i;
+      const int c = tid + NT * i;
       *reinterpret_cast<uint4*>(ks + (c / DC) * KLD + (c % DC) * 8) = kreg[i];
     }
     if (v_on) {
@@ -169,38 +173,49 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         sacc[rt] = mfma32(a, qf[s], sacc[rt]);
       }
     }
-    // ---- mask, running maximum
+    // ---- mask (only tiles that touch the diagonal or the window's edge), running maximum.
+    // Scores stay unscaled: the scale is positive, so the maximum can be taken first and the
+    // scale folded into the exponent's argument.
+    const bool edge = (kt * RB_PAGE + RB_PAGE - 1 > wave_min_pos) || (window > 0 && kt * RB_PAGE < wave_max_lo);
     float mx = -INFINITY;
+    if (edge) {
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int key = kt * RB_PAGE + rt * 32 + 8 * (e / 4) + 4 * g + (e % 4);
+          if (key > qpos || key < q_lo) sacc[rt][e] = -INFINITY;
+        }
+    }
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int key = kt * RB_PAGE + rt * 32 + 8 * (e / 4) + 4 * g + (e % 4);
-        float s = sacc[rt][e] * scale_log2;
-        if (key > qpos || key < q_lo) s = -INFINITY;
-        sacc[rt][e] = s;
-        mx = fmaxf(mx, s);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[rt][e]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale_log2;
     const float m_new = fmaxf(m_run, mx);
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float corr = exp2f(m_run - m_safe);          // m_run = -inf gives 0
     float lsum = 0.f;
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const float p = exp2f(sacc[rt][e] - m_safe);
+        const float p = __builtin_amdgcn_exp2f(fmaf(sacc[rt][e], scale_log2, -m_safe));
         sacc[rt][e] = p;
         lsum += p;
       }
     lsum += __shfl_xor(lsum, 32, 64);
-    l_run = l_run * corr + lsum;
+    // the accumulators are rescaled only when some query's maximum moved (rare after the
+    // first tiles)
+    if (__any(m_new != m_run)) {
+      const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);          // m_run = -inf gives 0
+      l_run *= corr;
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) oacc[i][e] *= corr;
+    }
+    l_run += lsum;
     m_run = m_new;
-#pragma unroll
-    for (int i = 0; i < D / 32; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) oacc[i][e] *= corr;
 
     // ---- O^T += V^T P^T.  Step (rt, mm) takes the 16 keys whose probabilities sit in
     // registers 8 mm .. 8 mm + 7 of row tile rt: for lane group g these are keys
@@ -250,19 +265,27 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
   RB_REQUIRE(window >= 0, "rb_attention_prefill_bf16: negative window");
   const int group = n_heads / n_kv_heads;
   const int gw = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
-  const int q_per_wg = 32 * (4 / gw);
+  // 8 waves (two per SIMD, which cover each other's softmax arithmetic) when the longest
+  // sequence gives them all queries; 4 for short steps
+  const int nw = max_q_len > 32 * (4 / gw) ? 8 : 4;
+  const int q_per_wg = 32 * (nw / gw);
   dim3 grid((max_q_len + q_per_wg - 1) / q_per_wg, n_kv_heads * (group / gw), n_seqs);
   RB_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "rb_attention_prefill_bf16: batch or head count too large");
   hipStream_t s = (hipStream_t)stream;
   const float sl2 = scale * LOG2E;
-  if (head_dim == 128)
-    attn_prefill_kernel<128><<<grid, 256, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
-                                                 (bf16_t*)out, cu_seqlens, past_len, block_table, bt_stride,
-                                                 n_heads, n_kv_heads, sl2, window, gw);
-  else
-    attn_prefill_kernel<64><<<grid, 256, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
-                                                (bf16_t*)out, cu_seqlens, past_len, block_table, bt_stride,
-                                                n_heads, n_kv_heads, sl2, window, gw);
+#define RB_PF(DV, NWV)                                                                                          \
+  attn_prefill_kernel<DV, NWV><<<grid, 64 * NWV, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages,              \
+                                                         (const bf16_t*)v_pages, (bf16_t*)out, cu_seqlens,      \
+                                                         past_len, block_table, bt_stride, n_heads, n_kv_heads, \
+                                                         sl2, window, gw)
+  if (head_dim == 128) {
+    if (nw == 8) RB_PF(128, 8);
+    else RB_PF(128, 4);
+  } else {
+    if (nw == 8) RB_PF(64, 8);
+    else RB_PF(64, 4);
+  }
+#undef RB_PF
   RB_LAUNCH_CHECK();
   return 0;
 }

@@ -37,12 +37,16 @@ struct bf16_t {
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 
-// round to nearest even; NaN stays NaN
+// round to nearest even, NaN stays NaN: the hardware's conversion (v_cvt_pk_bf16_f32)
+typedef __attribute__((ext_vector_type(2))) __bf16 rb_bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) float rb_f32x2_t;
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  union {
+    __bf16 b;
+    uint16_t u;
+  } r;
+  r.b = (__bf16)f;
+  return r.u;
 }
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
   bf16_t r;
@@ -50,7 +54,13 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
   return r;
 }
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+  union {
+    rb_bf16x2_t v;
+    uint32_t u;
+  } r;
+  const rb_f32x2_t f = {lo, hi};
+  r.v = __builtin_convertvector(f, rb_bf16x2_t);
+  return r.u;
 }
 
 template <typename T>
