@@ -198,10 +198,10 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int n
 // waves beat 8 at K = 4096, 8 beat 4 at K = 14336.
 template <int MB, int R, int EPI, typename TO>
 static int launch_skinny_u(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
-  constexpr int max_waves = (R * MB <= 4) ? 8 : 4;      // bounds the reduction buffer
+  constexpr int max_waves = (R * MB <= 4) ? 8 : (R * MB <= 8 ? 4 : 3);      // bounds the reduction buffer
   if (k % 128 == 0) {
     const int t = k / 128;
-    const int first_nw = k >= 8192 ? max_waves : 4;
+    const int first_nw = (k >= 8192 || max_waves < 4) ? max_waves : 4;
     for (int nw = g_tune_waves ? g_tune_waves : first_nw; nw >= 1; --nw) {
       if (t % nw != 0) continue;
       return launch_skinny<MB, R, 1, true, EPI, TO>(x, w, c, m, n, k, nw, k / nw, s);
@@ -225,7 +225,6 @@ static int dispatch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int
   else if (n >= 6144) r = 2;
   if (g_tune_r) r = g_tune_r;
   if (EPI == 1 && r < 2) r = 2;
-  if (mb >= 3 && r > 2) r = 2;
 #define RB_SK(MBV, RV) return launch_skinny_u<MBV, RV, EPI, TO>(x, w, c, m, n, k, s)
   if (mb == 1) {
     if (r == 4) RB_SK(1, 4);
@@ -236,9 +235,11 @@ static int dispatch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int
     if (r == 2) RB_SK(2, 2);
     if (EPI == 0) RB_SK(2, 1);
   } else if (mb == 3) {
+    if (r == 4) RB_SK(3, 4);
     if (r == 2) RB_SK(3, 2);
     if (EPI == 0) RB_SK(3, 1);
   } else {
+    if (r == 4) RB_SK(4, 4);
     if (r == 2) RB_SK(4, 2);
     if (EPI == 0) RB_SK(4, 1);
   }
