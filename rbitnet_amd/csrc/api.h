@@ -49,8 +49,11 @@ int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dty
 //               (16 gate rows, then the 16 up rows of the same columns); the result is
 //               silu(gate) * up, [M, N/2]
 // K must be a multiple of 8 (rows 16-byte aligned).
+// workspace: rb_gemm_workspace_floats(m, n, k, epilogue) floats (0: none, null allowed); contents do
+// not matter before or after.
+long long rb_gemm_workspace_floats(int m, int n, int k, int epilogue);
 int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
-                 void* stream);
+                 float* workspace, void* stream);
 
 // Causal attention of every token over its sequence's cache (keys 0..pos, or the last
 // `window` of them), any head_dim that is even and at most 256.

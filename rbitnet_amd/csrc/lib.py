@@ -64,7 +64,7 @@ class Kernels:
             "rb_rope_kv_write": [_P, _P, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
             "rb_swiglu": [_P, _P, _I, _I, _I, _P],
             "rb_gemm_generic": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
-            "rb_gemm_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "rb_gemm_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P],
             "rb_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_prefill_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_decode_bf16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
@@ -76,6 +76,8 @@ class Kernels:
             fn = getattr(L, name)
             fn.argtypes = args
             fn.restype = _I
+        L.rb_gemm_workspace_floats.argtypes = [_I, _I, _I, _I]
+        L.rb_gemm_workspace_floats.restype = ctypes.c_longlong
         L.rb_sample_workspace_bytes.argtypes = [_I, _I]
         L.rb_sample_workspace_bytes.restype = _I
         self.page_size = int(L.rb_page_size())
@@ -162,8 +164,10 @@ class Kernels:
         _check(a, "a", torch.bfloat16)
         _check(w, "w", torch.bfloat16, (n, k))
         _check(c, "c", None, (m, n // 2 if epilogue == 1 else n))
+        need = int(self._lib.rb_gemm_workspace_floats(m, n, k, int(epilogue)))
+        workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need else None
         self._ok(self._lib.rb_gemm_bf16(_ptr(a), _ptr(w), _ptr(c), dtype_code(c.dtype), int(epilogue), m, n, k,
-                                        self._stream()))
+                                        _ptr(workspace), self._stream()))
 
     def attention_generic(self, q, k_pages, v_pages, out, tok_pos, tok_seq, block_table, n_heads, n_kv, head_dim,
                           scale, window) -> None:

@@ -367,3 +367,30 @@ def test_attention_decode_fused_bf16(lib, n_heads, n_kv, d, window, n_splits, st
         for b in range(nb):
             page, off = int(bt[b, past[b] // 64]), past[b] % 64
             assert torch.equal(kp[page, :, off].cpu(), k_new[b]) and torch.equal(vp[page, :, off].cpu(), v_new[b])
+
+
+@pytest.mark.parametrize("m", [17, 31, 48, 64])
+@pytest.mark.parametrize("n,k,epi", [(4096, 1024, 0), (520, 512, 0), (200, 128, 0), (6144, 4096, 0), (672, 256, 1),
+                                     (8208 * 2, 384, 1)])
+def test_gemm_bf16_panel_shapes(lib, m, n, k, epi):
+    """17..64 tokens with K a multiple of 128: the kernel that shares the tokens through LDS,
+    with and without K split over workgroups (the workspace is filled with NaN first)."""
+    g = torch.Generator().manual_seed(m * 3 + n)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    if epi:
+        from rbitnet_amd.parts.linear import pack_gate_up
+        ff = n // 2
+        wg = (torch.randn(ff, k, generator=g) * 0.3).bfloat16()
+        wu = (torch.randn(ff, k, generator=g) * 0.3).bfloat16()
+        gate = a.double() @ wg.double().T
+        want = gate / (1 + torch.exp(-gate)) * (a.double() @ wu.double().T)
+        w = pack_gate_up(wg, wu, True)
+        out = torch.full((m, ff), float("nan"), device=DEV, dtype=torch.bfloat16)
+        tol = 1e-2
+    else:
+        w = torch.randn(n, k, generator=g).bfloat16()
+        want = a.double() @ w.double().T
+        out = torch.full((m, n), float("nan"), device=DEV, dtype=torch.float32)
+        tol = 2e-5
+    lib.gemm_bf16(a.to(DEV), w.to(DEV), out, epi)
+    assert _rel(out, want) < tol
