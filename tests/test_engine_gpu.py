@@ -57,6 +57,10 @@ def test_unequal_batches_with_slot_reuse(name, dtype):
     lengths = LENGTHS[name]
     eng = _engine(name, dtype, max_batch=len(lengths), max_tokens=64 * sum((n + 63) // 64 for n in lengths))
     for round_ in range(2):
+        # what earlier sequences left in the pages must not matter: poison all of it
+        for g in eng.cache.kv_groups:
+            g.k.fill_(float("nan"))
+            g.v.fill_(float("nan"))
         reqs = [tokens_for(name, n, 10 * round_ + i) for i, n in enumerate(lengths)]
         prompt_len = [max(1, len(r) - (3 + 5 * i)) for i, r in enumerate(reqs)]
         slots = [eng.alloc_slot() for _ in reqs]

@@ -394,3 +394,55 @@ def test_gemm_bf16_panel_shapes(lib, m, n, k, epi):
         tol = 2e-5
     lib.gemm_bf16(a.to(DEV), w.to(DEV), out, epi)
     assert _rel(out, want) < tol
+
+
+def test_attention_long_context(lib):
+    """Thousands of keys over many pages: decode with several split counts and a prompt step
+    on top of a long past (chunked prefill), against the plain computation."""
+    n_heads, n_kv, d = 8, 2, 128
+    dtype = torch.bfloat16
+    past, q_lens = [5000, 4097], [1, 1]
+    g, bt, tok_seq, tok_pos, total = _paged_setup(past, q_lens, n_kv, d, dtype, n_pages=160, seed=9)
+    k_full = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in total]
+    v_full = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in total]
+    q = (torch.randn(2, n_heads, d, generator=g) * 1.5).to(dtype)
+    kp, vp = _fill_pages(k_full, v_full, bt, 160, n_kv, d, dtype)
+    kp, vp = kp.to(DEV), vp.to(DEV)
+    scale = 1 / math.sqrt(d)
+    want = _attention_ref(q, k_full, v_full, tok_seq, tok_pos, n_heads, n_kv, scale, 0)
+    for n_splits in (1, 3, 16):
+        out = torch.full((2, n_heads * d), float("nan"), dtype=dtype, device=DEV)
+        ws = torch.empty(2 * n_heads * n_splits * (d + 2), device=DEV)
+        lib.attention_decode_bf16(q.to(DEV), kp, vp, out, tok_pos.to(DEV), bt.to(DEV), n_heads, n_kv, d, scale, 0,
+                                  n_splits, ws)
+        assert _rel(out, want) < 1e-2, n_splits
+    # a 100-token step on top of 4000 cached tokens
+    past, q_lens = [4000], [100]
+    g, bt, tok_seq, tok_pos, total = _paged_setup(past, q_lens, n_kv, d, dtype, n_pages=160, seed=10)
+    k_full = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in total]
+    v_full = [torch.randn(n, n_kv, d, generator=g).to(dtype) for n in total]
+    q = (torch.randn(100, n_heads, d, generator=g) * 1.5).to(dtype)
+    kp, vp = _fill_pages(k_full, v_full, bt, 160, n_kv, d, dtype)
+    out = torch.full((100, n_heads * d), float("nan"), dtype=dtype, device=DEV)
+    cu = torch.tensor([0, 100], dtype=torch.int32, device=DEV)
+    lib.attention_prefill_bf16(q.to(DEV), kp.to(DEV), vp.to(DEV), out, cu,
+                               torch.tensor(past, dtype=torch.int32, device=DEV), bt.to(DEV), 1, 100, n_heads, n_kv,
+                               d, scale, 0)
+    want = _attention_ref(q, k_full, v_full, tok_seq, tok_pos, n_heads, n_kv, scale, 0)
+    assert _rel(out, want) < 1.5e-2
+
+
+def test_sample_frequencies_follow_softmax(lib):
+    """20,000 draws with evenly spread uniform numbers: the frequency of every token is its
+    softmax probability at the given temperature (to within a draw or two)."""
+    g = torch.Generator().manual_seed(4)
+    vocab, n, temp = 50, 20000, 0.7
+    row = torch.randn(vocab, generator=g) * 2
+    logits = row[None, :].expand(n, vocab).contiguous().to(DEV)
+    us = ((torch.arange(n) + 0.5) / n).float().to(DEV)
+    temps = torch.full((n,), temp, device=DEV)
+    tokens = torch.empty(n, dtype=torch.int32, device=DEV)
+    lib.sample(logits, temps, us, tokens)
+    counts = torch.bincount(tokens.long().cpu(), minlength=vocab).double()
+    want = torch.softmax(row.double() / temp, 0) * n
+    assert float((counts - want).abs().max()) <= 2.0
