@@ -1,0 +1,167 @@
+"""Decode and prefill throughput of the engine at the Llama-3-8B shape, one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--no-points]
+    rbitnet bench   (the same options)
+
+A step is one decode step of the whole batch: the model's forward on one token per
+sequence from the cache, and the choice of the next tokens on the GPU.  Weights are
+random N(0, 0.02) bfloat16, token ids seeded uniform; prompts of 512 tokens are prefilled
+first, so the timed steps run at contexts from 512 upwards (the reference publishes no
+numbers, so `vs_baseline` is null).  One JSON line is printed.
+
+  value               decoded tokens per second at the default batch (8)
+  prefill             one prompt of 2,048 tokens: tokens/s, ms, fraction of the bf16 peak
+  roofline            bytes a decode step must read (weights once + live cache) / time
+  points              decode tokens/s at batch 1 and 64
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+PEAK_HBM = 8.0e12
+
+LLAMA3_8B = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "num_hidden_layers": 32,
+    "num_attention_heads": 32, "num_key_value_heads": 8, "intermediate_size": 14336, "vocab_size": 128256,
+    "rope_theta": 500000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 8192, "tie_word_embeddings": False,
+}
+PROMPT_LEN = 512
+NEW_TOKENS = 256
+PREFILL_TOKENS = 2048
+
+
+def _sync():
+    import torch
+    torch.cuda.synchronize()
+
+
+def matmul_flops_per_token(cfg) -> float:
+    e, f, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    hq, hk = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    d = cfg.get("head_dim") or e // hq
+    per_layer = 2 * (e * (hq + 2 * hk) * d + hq * d * e + 3 * e * f)
+    return per_layer * cfg["num_hidden_layers"], 2 * e * v
+
+
+def decode_run(engine, batch: int, steps: int, warmup: int, seed: int = 0):
+    """Prefill `batch` prompts of PROMPT_LEN tokens, then time `steps` decode steps."""
+    import numpy as np
+    import torch
+    rng = np.random.default_rng(seed)
+    vocab = engine.spec.vocab_size
+    slots = [engine.alloc_slot() for _ in range(batch)]
+    prompts = [[int(t) for t in rng.integers(0, vocab, size=PROMPT_LEN)] for _ in range(batch)]
+    # prompts go in groups so that a step's activations stay modest
+    group = max(1, 8192 // PROMPT_LEN)
+    last = []
+    for i in range(0, batch, group):
+        logits = engine.step([(s, p) for s, p in zip(slots[i:i + group], prompts[i:i + group])], "last")
+        last.extend(engine.sampler.sample(logits))
+    tokens = last
+    ctx0 = PROMPT_LEN
+    for _ in range(warmup):
+        tokens = engine.decode_step(slots, tokens)
+    _sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tokens = engine.decode_step(slots, tokens)
+    _sync()
+    dt = time.perf_counter() - t0
+    ctx_mean = ctx0 + warmup + (steps - 1) / 2.0 + 1
+    for s in slots:
+        engine.free_slot(s)
+    return dt, ctx_mean
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="bench")
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    args = ap.parse_args(argv)
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (this library has no multi-GPU path); --gpus {args.gpus} is not run")
+        return 2
+
+    import torch
+    from .engine import Engine
+
+    cfg = dict(LLAMA3_8B)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    layers = cfg["num_hidden_layers"]
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    ctx_cap = PROMPT_LEN + NEW_TOKENS + 64
+    max_tokens = max(max_batch * ctx_cap, PREFILL_TOKENS + 64)
+    engine = Engine.random(cfg, seed=0, dtype=dtype, std=0.02, norm_std=0.0, max_batch=max_batch,
+                                       max_tokens=max_tokens, max_seq_len=max(ctx_cap, PREFILL_TOKENS + 64))
+    _sync()
+
+    dt, ctx_mean = decode_run(engine, args.batch, args.steps, args.warmup)
+    ms = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+
+    hk = cfg["num_key_value_heads"]
+    d = cfg["hidden_size"] // cfg["num_attention_heads"]
+    esize = 2 if args.dtype == "bf16" else 4
+    kv_bytes_per_token = 2 * hk * d * esize * layers
+    step_bytes = engine.model.weight_bytes() + args.batch * ctx_mean * kv_bytes_per_token
+    achieved = step_bytes / (dt / args.steps)
+
+    out = {
+        "metric": "decode tok/s at batch 8 (Llama-3-8B shape)", "value": round(value, 2), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic: random N(0,0.02) weights, seeded uniform token ids",
+        "config": {
+            "model": "Llama-3-8B shape", "global_batch": args.batch, "seq_len": PROMPT_LEN + NEW_TOKENS,
+            "prompt_len": PROMPT_LEN, "parallelism": "single GPU", "layers": layers, "layers_full": full_layers,
+            "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": hk, "head_dim": d,
+            "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
+            "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
+            "context": cfg["max_position_embeddings"], "mean_context": round(ctx_mean, 1),
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM, 4)},
+    }
+
+    if not args.no_points:
+        # ---- prefill of one prompt of 2,048 tokens
+        import numpy as np
+        rng = np.random.default_rng(1)
+        prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=PREFILL_TOKENS)]
+        times = []
+        for i in range(4):
+            slot = engine.alloc_slot()
+            _sync()
+            t0 = time.perf_counter()
+            engine.step([(slot, prompt)], "last")
+            _sync()
+            times.append(time.perf_counter() - t0)
+            engine.free_slot(slot)
+        pt = min(times[1:])
+        layer_flops, head_flops = matmul_flops_per_token(cfg)
+        attn_flops = 4.0 * cfg["num_attention_heads"] * d * layers * (PREFILL_TOKENS * (PREFILL_TOKENS + 1) / 2.0)
+        flops = layer_flops * PREFILL_TOKENS + head_flops * 1 + attn_flops
+        out["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
+                          "frac": round(flops / pt / PEAK_FLOPS[args.dtype], 4)}
+        points = {}
+        for b in (1, 64):
+            steps = max(16, args.steps // 2)
+            dtb, _ = decode_run(engine, b, steps, max(4, args.warmup // 2), seed=b)
+            points[f"decode_b{b}"] = round(b * steps / dtb, 2)
+        out["points"] = points
+
+    print(json.dumps(out))
+    return 0
+

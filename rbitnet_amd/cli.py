@@ -8,6 +8,7 @@ with 1, main.rs:300-303).
     rbitnet random   --config config.json --out DIR [--seed 42] [--init-std 0.02] [--norm-std 0.02]
     rbitnet inspect  DIR_OR_FILE
     rbitnet replay   --model DIR --dtype D --out DIR --max-tokens N   < trace.jsonl
+    rbitnet bench    [--steps K] [--warmup W] [--batch B] [--layers L] [--no-points]
 
 Environment, as the reference's engine reads it (crates/bitnet-core/src/inference.rs:16-41):
 RBITNET_MODEL (default of --model; must not contain '..', inference.rs:44-53), RBITNET_TOY=1
@@ -145,6 +146,11 @@ def cmd_replay(args) -> int:
     return 0
 
 
+def cmd_bench(args) -> int:
+    from .benchmark import main as bench_main
+    return bench_main(args.rest)
+
+
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="rbitnet", description="rbitnet_amd: Llama-decoder generation on one MI355X")
     sub = ap.add_subparsers(dest="command", required=True)
@@ -184,10 +190,19 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--out", required=True)
     p.add_argument("--max-tokens", type=int, required=True)
     p.set_defaults(fn=cmd_replay)
+
+    b = sub.add_parser("bench", help="decode and prefill throughput at the Llama-3-8B shape (one JSON line)",
+                       add_help=False)
+    b.add_argument("rest", nargs=argparse.REMAINDER)
+    b.set_defaults(fn=cmd_bench)
     return ap
 
 
 def main(argv: Optional[List[str]] = None) -> int:
+    argv = list(sys.argv[1:] if argv is None else argv)
+    if argv and argv[0] == "bench":             # its options are the benchmark's own
+        from .benchmark import main as bench_main
+        return bench_main(argv[1:])
     args = build_parser().parse_args(argv)
     try:
         return args.fn(args)
