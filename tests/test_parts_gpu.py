@@ -260,3 +260,151 @@ def test_toy_mixer_and_mixed_layers(dtype, tol):
     eng.cache.check()
     # the windowed group gave pages back while the long sequence ran
     assert eng.cache.kv_groups[0].table.pool.n_free == eng.cache.n_pages
+
+
+# ---------------------------------------------------------------------------- other toy parts
+class HalfRotary(Part):
+    """Another position encoding, defined here: only the first half of each head's pairs is
+    rotated (the rest keeps angle 0), with frequencies of its own.  It is nothing but
+    another angle table for the existing kernels, the fused decode kernel included."""
+    graph_safe = True
+
+    def __init__(self, params, env):
+        self.env = env
+        d = int(params["head_dim"])
+        n = int(params["max_positions"])
+        inv = torch.zeros(d // 2, dtype=torch.float64)
+        inv[: d // 4] = 1.0 / (float(params["theta"]) ** (torch.arange(d // 4, dtype=torch.float64) * 4 / d))
+        self.inv = inv
+        ang = torch.arange(n, dtype=torch.float64)[:, None] * inv[None, :]
+        self.cos = torch.cos(ang).float().to(env.device) if env.lib is not None else None
+        self.sin = torch.sin(ang).float().to(env.device) if env.lib is not None else None
+
+    def rotation_tables(self):
+        return self.cos, self.sin, 0
+
+    def encode_and_store(self, qkv, q_out, k_pages, v_pages, ctx, block_table, n_heads, n_kv, head_dim):
+        self.env.lib.rope_kv_write(qkv, self.cos, self.sin, 0, q_out, k_pages, v_pages, ctx.tok_pos, ctx.tok_seq,
+                                   block_table, n_heads, n_kv, head_dim)
+
+
+class TopOneExperts(Part):
+    """A feed-forward with routing, defined here: a float32 router picks one of E small
+    SiLU-gated experts per token (torch operations; scratch sized by the step's tokens)."""
+
+    def __init__(self, params, env):
+        self.env, self.n_exp, self.ff, self.hidden = env, int(params["experts"]), int(params["ff"]), env.hidden_size
+
+    def tensor_specs(self):
+        specs = {"router.weight": TensorSpec((self.n_exp, self.hidden), role="gain", init="normal")}
+        for e in range(self.n_exp):
+            specs[f"experts.{e}.gate.weight"] = TensorSpec((self.ff, self.hidden))
+            specs[f"experts.{e}.up.weight"] = TensorSpec((self.ff, self.hidden))
+            specs[f"experts.{e}.down.weight"] = TensorSpec((self.hidden, self.ff))
+        return specs
+
+    def load(self, tensors):
+        self.w = tensors
+
+    def forward(self, h, ctx=None):
+        hf = h.float()
+        choice = (hf @ self.w["router.weight"].float().T).argmax(dim=1)
+        out = torch.zeros_like(hf)
+        for e in range(self.n_exp):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                x = hf[rows]
+                g = x @ self.w[f"experts.{e}.gate.weight"].float().T
+                u = x @ self.w[f"experts.{e}.up.weight"].float().T
+                out[rows] = (torch.nn.functional.silu(g) * u) @ self.w[f"experts.{e}.down.weight"].float().T
+        return out
+
+
+def _plain_other_parts(spec, tensors, tokens, inv):
+    w = {k: v.double().cpu() for k, v in tensors.items()}
+    x = P.embedding(w[spec.embedding_name], tokens)
+    margin = float("inf")
+    for layer in spec.layers:
+        pre = layer.prefix
+        m = layer.mixer
+        hq, hk, d = m["num_heads"], m["num_kv_heads"], m["head_dim"]
+        h = P.rmsnorm(x, w[f"{pre}.input_layernorm.weight"], layer.norm1["eps"])
+        q = P.linear(h, w[f"{pre}.self_attn.q_proj.weight"])
+        k = P.linear(h, w[f"{pre}.self_attn.k_proj.weight"])
+        v = P.linear(h, w[f"{pre}.self_attn.v_proj.weight"])
+        for pos in range(h.shape[0]):
+            for j in range(hq):
+                q[pos, j * d:(j + 1) * d] = P.rope(q[pos, j * d:(j + 1) * d], pos, inv)
+            for j in range(hk):
+                k[pos, j * d:(j + 1) * d] = P.rope(k[pos, j * d:(j + 1) * d], pos, inv)
+        x = x + P.linear(P.attention(q, k, v, hq, hk, None), w[f"{pre}.self_attn.o_proj.weight"])
+        h2 = P.rmsnorm(x, w[f"{pre}.post_attention_layernorm.weight"], layer.norm2["eps"])
+        logits = P.linear(h2, w[f"{pre}.mlp.router.weight"])
+        f = torch.zeros_like(x)
+        top = torch.topk(logits, 2, dim=1).values
+        margin = min(margin, float((top[:, 0] - top[:, 1]).min()))
+        for t in range(x.shape[0]):
+            e = int(logits[t].argmax())
+            f[t] = P.swiglu(h2[t:t + 1], w[f"{pre}.mlp.experts.{e}.gate.weight"], w[f"{pre}.mlp.experts.{e}.up.weight"],
+                            w[f"{pre}.mlp.experts.{e}.down.weight"])[0]
+        x = x + f
+    xn = P.rmsnorm(x, w[spec.final_norm_name], spec.final_norm["eps"])
+    return P.linear(xn, w[spec.head_name]), margin
+
+
+def test_toy_position_and_routed_feed_forward():
+    """Registered from the test, built by the framework, stepped whole, in pieces and as a
+    batch; head size 64 so that the matrix-core attention kernels (and the fused decode
+    kernel with the toy's angle table) run."""
+    import rbitnet_amd
+    from rbitnet_amd.engine.model import expected_tensors
+    from rbitnet_amd.parts import register_feed_forward, register_position
+    from rbitnet_amd.weights import random_tensors
+    register_position("half_rotary", HalfRotary)
+    register_feed_forward("top_one_experts", TopOneExperts)
+    hidden, vocab, d = 64, 70, 64
+    norm = PartSpec("rmsnorm", {"size": hidden, "eps": 1e-5})
+    pos = PartSpec("half_rotary", {"head_dim": d, "theta": 100.0, "max_positions": 512})
+    att = {"num_heads": 2, "num_kv_heads": 1, "head_dim": d, "scale": d ** -0.5, "window": None, "cache_from": None,
+           "position": pos}
+    layers = [LayerSpec(f"blocks.{i}", "prenorm", PartSpec("attention", att),
+                        PartSpec("top_one_experts", {"experts": 3, "ff": 40}), norm, norm) for i in range(2)]
+    spec = ModelSpec(architecture="ToyForTests", hidden_size=hidden, vocab_size=vocab, max_positions=512,
+                     embedding_name="embed.weight", layers=layers, final_norm=norm,
+                     final_norm_name="final_norm.weight", head_name="head.weight")
+    expected = expected_tensors(spec)
+    assert "blocks.1.mlp.experts.2.down.weight" in expected
+    tensors = dict(random_tensors(expected, seed=6, std=0.15, norm_std=0.05, dtype=torch.bfloat16))
+    for name in tensors:
+        if name.endswith("router.weight"):
+            tensors[name] = tensors[name] * 8          # clear-cut choices, so that rounding cannot flip one
+    eng = rbitnet_amd.Engine.from_spec(spec, tensors, dtype="bfloat16", max_tokens=64 * 8, max_batch=2)
+    assert not eng.use_graphs                          # the routed feed-forward reads device data on the host
+    inv = HalfRotary(pos.params, BuildEnv(hidden, torch.float32, torch.device("cpu"), None)).inv
+    # a router's choice between two nearly equal logits may fall either way in bfloat16: take
+    # sequences whose choices are all clear-cut in the plain computation
+    g = torch.Generator().manual_seed(2)
+    seqs, want = [], []
+    for n in (90, 20):
+        for _ in range(20):
+            s = torch.randint(0, vocab, (n,), generator=g).tolist()
+            logits, margin = _plain_other_parts(spec, tensors, s, inv)
+            if margin > 0.15:
+                break
+        else:
+            pytest.fail("no sequence with clear-cut routing found")
+        seqs.append(s)
+        want.append(logits)
+    slots = [eng.alloc_slot() for _ in seqs]
+    cut = [len(s) - 4 for s in seqs]
+    logits = eng.step([(sl, s[:c]) for sl, s, c in zip(slots, seqs, cut)], "all")
+    off = 0
+    for s, c, w in zip(seqs, cut, want):
+        assert _rel(logits[off:off + c], w[:c]) < 4e-2
+        off += c
+    for j in range(4):
+        logits = eng.step([(sl, [s[c + j]]) for sl, s, c in zip(slots, seqs, cut)], "last")
+        for i, (c, w) in enumerate(zip(cut, want)):
+            assert _rel(logits[i:i + 1], w[c + j:c + j + 1]) < 4e-2
+    for sl in slots:
+        eng.free_slot(sl)
