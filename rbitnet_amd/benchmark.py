@@ -29,6 +29,21 @@ LLAMA3_8B = {
     "num_attention_heads": 32, "num_key_value_heads": 8, "intermediate_size": 14336, "vocab_size": 128256,
     "rope_theta": 500000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 8192, "tie_word_embeddings": False,
 }
+# the other shapes the baseline names (configs[3] and [4]); chosen with --model
+LLAMA2_7B = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "num_hidden_layers": 32,
+    "num_attention_heads": 32, "num_key_value_heads": 32, "intermediate_size": 11008, "vocab_size": 32000,
+    "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 4096, "tie_word_embeddings": False,
+}
+LLAMA31_70B = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 8192, "num_hidden_layers": 80,
+    "num_attention_heads": 64, "num_key_value_heads": 8, "intermediate_size": 28672, "vocab_size": 128256,
+    "rope_theta": 500000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 8192, "tie_word_embeddings": False,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+}
+MODELS = {"llama3_8b": ("Llama-3-8B shape", LLAMA3_8B), "llama2_7b": ("Llama-2-7B shape", LLAMA2_7B),
+          "llama31_70b": ("Llama-3.1-70B shape", LLAMA31_70B)}
 PROMPT_LEN = 512
 NEW_TOKENS = 256
 PREFILL_TOKENS = 2048
@@ -47,22 +62,26 @@ def matmul_flops_per_token(cfg) -> float:
     return per_layer * cfg["num_hidden_layers"], 2 * e * v
 
 
-def decode_run(engine, batch: int, steps: int, warmup: int, seed: int = 0):
-    """Prefill `batch` prompts of PROMPT_LEN tokens, then time `steps` decode steps."""
+def decode_run(engine, batch: int, steps: int, warmup: int, seed: int = 0, prompt_len=PROMPT_LEN):
+    """Prefill `batch` prompts of `prompt_len` tokens (a pair (lo, hi): lengths drawn
+    uniformly from lo..hi), then time `steps` decode steps."""
     import numpy as np
-    import torch
     rng = np.random.default_rng(seed)
     vocab = engine.spec.vocab_size
     slots = [engine.alloc_slot() for _ in range(batch)]
-    prompts = [[int(t) for t in rng.integers(0, vocab, size=PROMPT_LEN)] for _ in range(batch)]
+    if isinstance(prompt_len, tuple):
+        lens = [int(n) for n in rng.integers(prompt_len[0], prompt_len[1] + 1, size=batch)]
+    else:
+        lens = [prompt_len] * batch
+    prompts = [[int(t) for t in rng.integers(0, vocab, size=n)] for n in lens]
     # prompts go in groups so that a step's activations stay modest
-    group = max(1, 8192 // PROMPT_LEN)
+    group = max(1, 8192 // max(lens))
     last = []
     for i in range(0, batch, group):
         logits = engine.step([(s, p) for s, p in zip(slots[i:i + group], prompts[i:i + group])], "last")
         last.extend(engine.sampler.sample(logits))
     tokens = last
-    ctx0 = PROMPT_LEN
+    ctx0 = sum(lens) / batch
     for _ in range(warmup):
         tokens = engine.decode_step(slots, tokens)
     _sync()
@@ -86,6 +105,10 @@ def main(argv=None) -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    ap.add_argument("--model", default="llama3_8b", choices=sorted(MODELS),
+                    help="shape to measure (default: the baseline's configs[2])")
+    ap.add_argument("--prompt-len", default=str(PROMPT_LEN),
+                    help="context at which decoding starts; LO,HI draws unequal lengths uniformly")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (this library has no multi-GPU path); --gpus {args.gpus} is not run")
@@ -94,20 +117,26 @@ def main(argv=None) -> int:
     import torch
     from .engine import Engine
 
-    cfg = dict(LLAMA3_8B)
+    if "," in args.prompt_len:
+        lo, hi = (int(v) for v in args.prompt_len.split(","))
+        prompt_len, longest = (lo, hi), hi
+    else:
+        prompt_len = longest = int(args.prompt_len)
+    model_name, base = MODELS[args.model]
+    cfg = dict(base)
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     layers = cfg["num_hidden_layers"]
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     max_batch = max(args.batch, 1 if args.no_points else 64)
-    ctx_cap = PROMPT_LEN + NEW_TOKENS + 64
+    ctx_cap = longest + max(NEW_TOKENS, args.steps + args.warmup) + 64
     max_tokens = max(max_batch * ctx_cap, PREFILL_TOKENS + 64)
     engine = Engine.random(cfg, seed=0, dtype=dtype, std=0.02, norm_std=0.0, max_batch=max_batch,
                                        max_tokens=max_tokens, max_seq_len=max(ctx_cap, PREFILL_TOKENS + 64))
     _sync()
 
-    dt, ctx_mean = decode_run(engine, args.batch, args.steps, args.warmup)
+    dt, ctx_mean = decode_run(engine, args.batch, args.steps, args.warmup, prompt_len=prompt_len)
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
 
@@ -119,13 +148,13 @@ def main(argv=None) -> int:
     achieved = step_bytes / (dt / args.steps)
 
     out = {
-        "metric": "decode tok/s at batch 8 (Llama-3-8B shape)", "value": round(value, 2), "unit": "tokens/s",
+        "metric": f"decode tok/s at batch {args.batch} ({model_name})", "value": round(value, 2), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic: random N(0,0.02) weights, seeded uniform token ids",
         "config": {
-            "model": "Llama-3-8B shape", "global_batch": args.batch, "seq_len": PROMPT_LEN + NEW_TOKENS,
-            "prompt_len": PROMPT_LEN, "parallelism": "single GPU", "layers": layers, "layers_full": full_layers,
+            "model": model_name, "global_batch": args.batch, "seq_len": longest + NEW_TOKENS,
+            "prompt_len": args.prompt_len if "," in args.prompt_len else longest, "parallelism": "single GPU", "layers": layers, "layers_full": full_layers,
             "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": hk, "head_dim": d,
             "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
             "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
@@ -158,7 +187,7 @@ def main(argv=None) -> int:
         points = {}
         for b in (1, 64):
             steps = max(16, args.steps // 2)
-            dtb, _ = decode_run(engine, b, steps, max(4, args.warmup // 2), seed=b)
+            dtb, _ = decode_run(engine, b, steps, max(4, args.warmup // 2), seed=b, prompt_len=prompt_len)
             points[f"decode_b{b}"] = round(b * steps / dtb, 2)
         out["points"] = points
 

@@ -20,7 +20,7 @@ import torch
 from ..cache import PAGE_SIZE, Cache, pages_for
 from ..config import load_config
 from ..errors import CacheError, ConfigError, InferenceError, KernelError
-from ..weights import DEFAULT_SEED, load_weights, random_tensors
+from ..weights import DEFAULT_SEED, RandomTensors, load_weights
 from .context import StepContext
 from .model import Model
 
@@ -102,7 +102,7 @@ class Engine:
         inference.rs:24-36)."""
         def tensors_for(model: Model, cfg):
             store = torch.bfloat16 if model.dtype == torch.bfloat16 else torch.float32
-            return dict(random_tensors(model.expected, seed, std, norm_std, store, device))
+            return RandomTensors(model.expected, seed, std, norm_std, store, device)
 
         return cls._build(config, tensors_for, dtype, max_tokens, max_batch, max_seq_len, device, generic_only)
 

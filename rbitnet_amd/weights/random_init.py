@@ -12,6 +12,7 @@ from __future__ import annotations
 import hashlib
 import json
 import os
+from collections.abc import Mapping
 from typing import Any, Dict, Iterator, Optional, Tuple
 
 import torch
@@ -49,6 +50,24 @@ def random_tensors(expected: Dict[str, TensorSpec], seed: int, std: float = 0.02
                    dtype: torch.dtype = torch.bfloat16, device: Any = "cpu") -> Iterator[Tuple[str, torch.Tensor]]:
     for name, spec in expected.items():
         yield name, random_tensor(name, spec, seed, std, norm_std, dtype, device)
+
+
+class RandomTensors(Mapping):
+    """name -> tensor, each drawn when it is asked for and not kept: a model far
+    larger than its biggest tensor can be filled without holding a second copy."""
+
+    def __init__(self, expected: Dict[str, TensorSpec], seed: int, std: float = 0.02, norm_std: float = 0.02,
+                 dtype: torch.dtype = torch.bfloat16, device: Any = "cpu"):
+        self._expected, self._args = expected, (seed, std, norm_std, dtype, device)
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        return random_tensor(name, self._expected[name], *self._args)
+
+    def __iter__(self):
+        return iter(self._expected)
+
+    def __len__(self) -> int:
+        return len(self._expected)
 
 
 def write_random_model(folder: str, config: Any, seed: int = DEFAULT_SEED, std: float = 0.02,
