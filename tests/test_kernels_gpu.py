@@ -85,6 +85,32 @@ def test_gemm_bf16_gated(lib, m, ff, k):
     assert _rel(out, want) < 1e-2
 
 
+@pytest.mark.parametrize("m,n,k,gated", [(513, 300, 128, False), (700, 14000, 192, False), (700, 14000, 64, False),
+                                         (257, 41000, 320, False), (600, 14016, 128, True), (130, 96, 64, True)])
+def test_gemm_bf16_tiles_loaded_straight_into_lds(lib, m, n, k, gated):
+    """K a multiple of 64 and more than 64 tokens: the kernels whose tiles go from memory into
+    LDS without passing registers, with both tile sizes, partial tiles at both edges, and as
+    few K tiles as one (fewer than the stages of the pipeline)."""
+    from rbitnet_amd.parts.linear import pack_gate_up
+    g = torch.Generator().manual_seed(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    if gated:
+        ff = n // 2
+        wg = (torch.randn(ff, k, generator=g) * 0.3).bfloat16()
+        wu = (torch.randn(ff, k, generator=g) * 0.3).bfloat16()
+        gate = x.double() @ wg.double().T
+        want = gate / (1 + torch.exp(-gate)) * (x.double() @ wu.double().T)
+        out = torch.full((m, ff), float("nan"), device=DEV, dtype=torch.bfloat16)
+        lib.gemm_bf16(x.to(DEV), pack_gate_up(wg, wu, True).to(DEV), out, 1)
+        assert _rel(out, want) < 1e-2
+    else:
+        w = torch.randn(n, k, generator=g).bfloat16()
+        want = x.double() @ w.double().T
+        out = torch.full((m, n), float("nan"), device=DEV, dtype=torch.float32)
+        lib.gemm_bf16(x.to(DEV), w.to(DEV), out, 0)
+        assert _rel(out, want) < 2e-5
+
+
 # ------------------------------------------------------------------------ elementwise
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_embed_gather(lib, dtype):
