@@ -413,140 +413,8 @@ static bool try_resident(const bf16_t* x, const bf16_t* w, void* c, int m, int n
   return true;
 }
 
-// =============================================================================== panel (16 < M <= 64)
-// With up to 64 tokens the token operand is too large to be read again by every wave from
-// L2 (it would outweigh W) and too large for registers.  Here a workgroup of 8 waves owns 128
-// rows of W (16 per wave) and a slice of K; the tokens' 128-deep chunk of that slice goes
-// through LDS once for all 8 waves (double-buffered, next chunk in flight in registers), W
-// goes from memory straight into MFMA operands.  Small N: K is also split over workgroups
-// (grid.y) and each writes its partial sums to its own [M, N] slab of a workspace, which
-// gemm_sum_slabs_kernel adds up in a fixed order.
-#define PN_LD 136          // bf16 elements per LDS row: 128 + 8 of padding
-
-template <int MB, int EPI, typename TO>
-__global__ __launch_bounds__(512) void gemm_panel_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                         TO* __restrict__ c, float* __restrict__ slabs, int m, int n,
-                                                         int k, int k_per_wg) {
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][16 * MB][PN_LD];
-  __shared__ float gate_s[EPI == 1 ? 4 : 1][EPI == 1 ? MB * 4 : 1][64];
-  constexpr int XQ = (256 * MB + 511) / 512;      // 16-byte pieces of a token chunk per thread
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 15, kq = lane >> 4;
-  const int row0 = blockIdx.x * 128 + wave * 16;
-  const int k_begin = blockIdx.y * k_per_wg;
-  const int chunks = k_per_wg / 128;
-  int wr = row0 + r;
-  if (wr > n - 1) wr = n - 1;                     // such rows are never stored
-  const bf16_t* wrow = w + (size_t)wr * k + k_begin + 8 * kq;
-
-  uint4 xreg[XQ];
-  auto load_x = [&](int ch) {
-#pragma unroll
-    for (int i = 0; i < XQ; ++i) {
-      const int q = tid + 512 * i;                // piece q: token q / 16, 16-byte column q % 16
-      int row = q / 16;
-      if (row > m - 1) row = m - 1;
-      xreg[i] = load16(x + (size_t)row * k + k_begin + ch * 128 + (q % 16) * 8);
-    }
-  };
-  auto store_x = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < XQ; ++i) {
-      const int q = tid + 512 * i;
-      if (q < 256 * MB) *reinterpret_cast<uint4*>(&xs[buf][q / 16][(q % 16) * 8]) = xreg[i];
-    }
-  };
-  Frag8 a0[4], a1[4];
-  auto load_w = [&](Frag8* a, int ch) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) a[j].u = load16(wrow + ch * 128 + 32 * j);
-  };
-  f32x4_t acc[MB];
-#pragma unroll
-  for (int cb = 0; cb < MB; ++cb) acc[cb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  auto multiply = [&](const Frag8* a, int buf) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int cb = 0; cb < MB; ++cb) {
-        Frag8 b;
-        b.u = *reinterpret_cast<const uint4*>(&xs[buf][16 * cb + r][32 * j + 8 * kq]);
-        acc[cb] = mfma16(a[j], b, acc[cb]);
-      }
-  };
-
-  load_x(0);
-  load_w(a0, 0);
-  store_x(0);
-  __syncthreads();
-  int ch = 0;
-  for (; ch + 2 <= chunks - 1; ch += 2) {         // chunks ch + 1 and ch + 2 exist: unconditional loads
-    load_x(ch + 1);
-    load_w(a1, ch + 1);
-    multiply(a0, 0);
-    store_x(1);
-    __syncthreads();
-    load_x(ch + 2);
-    load_w(a0, ch + 2);
-    multiply(a1, 1);
-    store_x(0);
-    __syncthreads();
-  }
-  if (ch + 1 <= chunks - 1) {
-    load_x(ch + 1);
-    load_w(a1, ch + 1);
-    multiply(a0, 0);
-    store_x(1);
-    __syncthreads();
-    multiply(a1, 1);
-  } else {
-    multiply(a0, 0);
-  }
-
-  // ---- lane holds, per cb: token 16 cb + r, W rows row0 + 4 kq + 0..3
-  if (EPI == 0) {
-    float* slab = slabs ? slabs + (size_t)blockIdx.y * m * n : nullptr;
-#pragma unroll
-    for (int cb = 0; cb < MB; ++cb) {
-      const int mm = 16 * cb + r;
-      const int nn = row0 + 4 * kq;
-      if (mm >= m) continue;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (nn + i >= n) continue;
-        if (slab)
-          slab[(size_t)mm * n + nn + i] = acc[cb][i];
-        else
-          Num<TO>::store(c + (size_t)mm * n + nn + i, acc[cb][i]);
-      }
-    }
-  } else {
-    // even waves hold gate tiles, odd waves the up tiles of the same columns
-    __syncthreads();
-    if ((wave & 1) == 0) {
-#pragma unroll
-      for (int cb = 0; cb < MB; ++cb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) gate_s[wave >> 1][cb * 4 + i][lane] = acc[cb][i];
-    }
-    __syncthreads();
-    if (wave & 1) {
-      const int half_n = n / 2;
-#pragma unroll
-      for (int cb = 0; cb < MB; ++cb) {
-        const int mm = 16 * cb + r;
-        const int nn = (row0 - 16) / 2 + 4 * kq;
-        if (mm >= m) continue;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (nn + i < half_n)
-            Num<TO>::store(c + (size_t)mm * half_n + nn + i,
-                           silu_f32(gate_s[wave >> 1][cb * 4 + i][lane]) * acc[cb][i]);
-      }
-    }
-  }
-}
-
+// Adds up the [M, N] slabs of partial sums that the K slices of a product wrote, in slice
+// order (the same order whatever else runs), and converts to the output type.
 template <typename TO>
 __global__ void gemm_sum_slabs_kernel(const float* __restrict__ slabs, TO* __restrict__ c, int parts, size_t count) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -554,57 +422,6 @@ __global__ void gemm_sum_slabs_kernel(const float* __restrict__ slabs, TO* __res
   float v = 0.f;
   for (int p = 0; p < parts; ++p) v += slabs[(size_t)p * count + i];
   Num<TO>::store(c + i, v);
-}
-
-static int g_panel_parts = 0;
-extern "C" void rb_tune_panel_parts(int p) { g_panel_parts = p; }      // experiments only; 0 = built-in
-
-// Into how many K slices the panel kernel cuts a product (1: no workspace needed).
-static int panel_parts(int m, int n, int k, int epilogue) {
-  if (m <= 16 || m > 64 || k % 128 != 0) return 0;          // not a panel product
-  const int tiles = (n + 127) / 128;
-  if (epilogue == 1 || tiles >= 200) return 1;
-  const int t = k / 128;
-  if (g_panel_parts && t % g_panel_parts == 0) return g_panel_parts;
-  // more slices fill more compute units, but every slice writes and re-reads an [M, N] slab:
-  // keep that traffic (8 bytes per slab element) under half of W's (2 N K bytes), the slices
-  // at 8 and the workgroups at about 320 (measured at M = 24..64 on the 4096- and 6144-row
-  // products of Llama-3-8B)
-  int cap = k / (8 * m);
-  if (cap > 8) cap = 8;
-  if (cap < 1) cap = 1;
-  int best = 1;
-  for (int p = 1; p <= t && p <= cap; ++p) {
-    if (t % p != 0 || t / p < 2) continue;                  // equal slices of at least 2 chunks
-    if ((long long)tiles * p <= 320) best = p;
-  }
-  return best;
-}
-
-extern "C" long long rb_gemm_workspace_floats(int m, int n, int k, int epilogue) {
-  const int p = panel_parts(m, n, k, epilogue);
-  return p > 1 ? (long long)p * m * n : 0;
-}
-
-template <int EPI, typename TO>
-static int launch_panel(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int m, int n, int k,
-                        hipStream_t s) {
-  const int parts = panel_parts(m, n, k, EPI);
-  RB_REQUIRE(parts >= 1, "rb_gemm_bf16: internal: not a panel product");
-  RB_REQUIRE(parts == 1 || workspace != nullptr, "rb_gemm_bf16: M=%d N=%d K=%d needs a workspace of %lld floats", m, n,
-             k, (long long)parts * m * n);
-  const int mb = (m + 15) / 16;
-  dim3 grid((n + 127) / 128, parts);
-  float* slabs = parts > 1 ? workspace : nullptr;
-  const int kpw = k / parts;
-  if (mb == 2) gemm_panel_kernel<2, EPI, TO><<<grid, 512, 0, s>>>(x, w, (TO*)c, slabs, m, n, k, kpw);
-  else if (mb == 3) gemm_panel_kernel<3, EPI, TO><<<grid, 512, 0, s>>>(x, w, (TO*)c, slabs, m, n, k, kpw);
-  else gemm_panel_kernel<4, EPI, TO><<<grid, 512, 0, s>>>(x, w, (TO*)c, slabs, m, n, k, kpw);
-  if (parts > 1) {
-    const size_t count = (size_t)m * n;
-    gemm_sum_slabs_kernel<TO><<<(unsigned)((count + 255) / 256), 256, 0, s>>>(slabs, (TO*)c, parts, count);
-  }
-  return 0;
 }
 
 // =============================================================================== tiled
@@ -838,7 +655,8 @@ __device__ __forceinline__ void load_to_lds16(const bf16_t* base, uint32_t byte_
 template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO>
 __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(const bf16_t* __restrict__ x,
                                                        const bf16_t* __restrict__ w, TO* __restrict__ c,
-                                                       int m, int n, int k, int m_tiles, int n_tiles) {
+                                                       float* __restrict__ slabs, int m, int n, int k, int m_tiles,
+                                                       int n_tiles, int k_tiles) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int TN = WN / 32, TM = WM / 32;
   constexpr int WAVES_N = BN / WN;
@@ -895,9 +713,10 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
     xoff[i] = ((uint32_t)grow * (uint32_t)k + chunk * 8) * 2u;
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;      // LDS byte address of stage 0
+  const int kt0 = blockIdx.y * k_tiles;                    // this workgroup's slice of K: k_tiles tiles from here
   auto issue = [&](int kt) {
     const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
-    const uint32_t kbytes = (uint32_t)kt * (BK * 2);
+    const uint32_t kbytes = (uint32_t)(kt0 + kt) * (BK * 2);
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i)
       load_to_lds16(wtile, woff[i] + kbytes, stage + (uint32_t)(wave + NWAVES * i) * 1024u);
@@ -932,7 +751,6 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
     }
   };
 
-  const int k_tiles = k / BK;
 #pragma unroll
   for (int s = 0; s < S - 1; ++s)
     if (s < k_tiles) issue(s);
@@ -954,11 +772,15 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
       if (mm >= m) continue;
       const int nbase = n0 + wn0 + 32 * i;
       if (EPI == 0) {
+        // a slice of K: partial sums go to this slice's [M, N] slab, to be added up in a fixed order
+        float* slab = slabs ? slabs + ((size_t)blockIdx.y * m + mm) * n : nullptr;
         TO* dst = c + (size_t)mm * n;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int nn = nbase + 8 * (e / 4) + 4 * g + (e % 4);
-          if (nn < n) Num<TO>::store(dst + nn, acc[i][j][e]);
+          if (nn >= n) continue;
+          if (slab) slab[nn] = acc[i][j][e];
+          else Num<TO>::store(dst + nn, acc[i][j][e]);
         }
       } else {
         const int half_n = n / 2;
@@ -973,8 +795,11 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
 }
 
 template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO>
-static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
+static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s,
+                          int parts = 1, float* slabs = nullptr) {
   const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
+  RB_REQUIRE(parts >= 1 && (k / BK) % parts == 0 && (parts == 1 || (slabs && EPI == 0)),
+             "rb_gemm_bf16: internal: bad K split %d", parts);
   const long long tiles = (long long)m_tiles * n_tiles;
   RB_REQUIRE(tiles < (1LL << 30), "rb_gemm_bf16: too many tiles");
   RB_REQUIRE(k % BK == 0, "rb_gemm_bf16: the direct-to-LDS kernel needs K=%d to be a multiple of %d", k, BK);
@@ -989,9 +814,59 @@ static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int 
     RB_REQUIRE(e == hipSuccess, "rb_gemm_bf16: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     configured = true;
   }
-  const int grid = (int)((tiles + 7) / 8 * 8);
-  kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, m, n, k, m_tiles, n_tiles);
+  const dim3 grid((unsigned)((tiles + 7) / 8 * 8), (unsigned)parts);
+  kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, parts > 1 ? slabs : nullptr, m, n, k, m_tiles,
+                                                      n_tiles, k / BK / parts);
+  if (parts > 1) {
+    const size_t count = (size_t)m * n;
+    gemm_sum_slabs_kernel<TO><<<(unsigned)((count + 255) / 256), 256, 0, s>>>(slabs, (TO*)c, parts, count);
+  }
   return 0;
+}
+
+// ------------------------------------------------------------------ 17 .. 64 tokens, K % 64 == 0
+// The same kernel with one token tile: W streams through LDS three stages deep, two
+// workgroups per compute unit.  Few rows of W: K is also cut into slices over workgroups
+// (grid.y); each slice writes its partial sums to its own [M, N] slab of a workspace, and
+// gemm_sum_slabs_kernel adds them up in a fixed order.
+static int g_stream_parts = 0;
+extern "C" void rb_tune_stream_parts(int parts) { g_stream_parts = parts; }      // experiments only; 0 = built-in
+
+static int stream_parts(int m, int n, int k, int epilogue) {
+  if (m <= 16 || m > 64 || k % 64 != 0 || (long long)k * 256 >= (1LL << 32)) return 0;      // not for this kernel
+  if (epilogue == 1) return 1;
+  const int tiles = (n + 127) / 128;
+  const int kt = k / 64;
+  if (g_stream_parts && kt % g_stream_parts == 0) return g_stream_parts;
+  // every slice writes and re-reads an [M, N] slab (8 bytes per element): keep that under half
+  // of W's bytes, the slices at 16 and at least 4 tiles deep, the workgroups at one per compute
+  // unit (more slices cost more in slabs than they gain: measured on N = 4096 and 6144)
+  int cap = k / (8 * m);
+  if (cap > 16) cap = 16;
+  int best = 1;
+  for (int p = 1; p <= cap; ++p) {
+    if (kt % p != 0 || kt / p < 4) continue;
+    if ((long long)tiles * p <= 256) best = p;
+  }
+  return best;
+}
+
+static int g_use_stream = 1;
+extern "C" void rb_tune_use_stream(int on) { g_use_stream = on; }      // experiments only
+
+extern "C" long long rb_gemm_workspace_floats(int m, int n, int k, int epilogue) {
+  const int p = g_use_stream ? stream_parts(m, n, k, epilogue) : 0;
+  return p > 1 ? (long long)p * m * n : 0;
+}
+
+template <int EPI, typename TO>
+static int launch_stream(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int m, int n, int k,
+                         hipStream_t s) {
+  const int parts = stream_parts(m, n, k, EPI);
+  RB_REQUIRE(parts >= 1, "rb_gemm_bf16: internal: not a product for the streaming kernel");
+  RB_REQUIRE(parts == 1 || workspace != nullptr, "rb_gemm_bf16: M=%d N=%d K=%d needs a workspace of %lld floats", m, n,
+             k, (long long)parts * m * n);
+  return launch_dma_cfg<128, 64, 32, 64, 64, 3, EPI, TO>(x, w, c, m, n, k, s, parts, workspace);
 }
 
 static int g_tile_cfg = 0;
@@ -1048,9 +923,6 @@ static int launch_tiled(const bf16_t* x, const bf16_t* w, void* c, int m, int n,
 static int g_use_resident = 1;
 extern "C" void rb_tune_use_resident(int on) { g_use_resident = on; }
 
-static int g_use_panel = 1;
-extern "C" void rb_tune_use_panel(int on) { g_use_panel = on; }
-
 extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out, int epilogue, int m, int n,
                             int k, float* workspace, void* stream) {
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_bf16: bad sizes M=%d N=%d K=%d", m, n, k);
@@ -1065,13 +937,13 @@ extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out
   int rc = 0;
   if (m <= 64) {
     bool done = false;
-    if (g_use_panel && panel_parts(m, n, k, epilogue) >= 1 && (epilogue == 0 || n % 32 == 0)) {
+    if (g_use_stream && stream_parts(m, n, k, epilogue) >= 1) {
       if (epilogue == 0)
-        rc = dtype_out == RB_F32 ? launch_panel<0, float>(xa, wa, c, workspace, m, n, k, s)
-                                 : launch_panel<0, bf16_t>(xa, wa, c, workspace, m, n, k, s);
+        rc = dtype_out == RB_F32 ? launch_stream<0, float>(xa, wa, c, workspace, m, n, k, s)
+                                 : launch_stream<0, bf16_t>(xa, wa, c, workspace, m, n, k, s);
       else
-        rc = dtype_out == RB_F32 ? launch_panel<1, float>(xa, wa, c, workspace, m, n, k, s)
-                                 : launch_panel<1, bf16_t>(xa, wa, c, workspace, m, n, k, s);
+        rc = dtype_out == RB_F32 ? launch_stream<1, float>(xa, wa, c, workspace, m, n, k, s)
+                                 : launch_stream<1, bf16_t>(xa, wa, c, workspace, m, n, k, s);
       done = true;
     }
     // many rows of W and at most 16 tokens: the kernel that keeps the tokens in registers

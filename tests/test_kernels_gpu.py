@@ -396,11 +396,11 @@ def test_attention_decode_fused_bf16(lib, n_heads, n_kv, d, window, n_splits, st
 
 
 @pytest.mark.parametrize("m", [17, 31, 48, 64])
-@pytest.mark.parametrize("n,k,epi", [(4096, 1024, 0), (520, 512, 0), (200, 128, 0), (6144, 4096, 0), (672, 256, 1),
-                                     (8208 * 2, 384, 1)])
-def test_gemm_bf16_panel_shapes(lib, m, n, k, epi):
-    """17..64 tokens with K a multiple of 128: the kernel that shares the tokens through LDS,
-    with and without K split over workgroups (the workspace is filled with NaN first)."""
+@pytest.mark.parametrize("n,k,epi", [(4096, 1024, 0), (520, 512, 0), (200, 128, 0), (100, 64, 0), (333, 192, 0),
+                                     (6144, 4096, 0), (672, 256, 1), (8208 * 2, 384, 1)])
+def test_gemm_bf16_17_to_64_tokens(lib, m, n, k, epi):
+    """17..64 tokens with K a multiple of 64: one token tile, W streamed through LDS, with
+    and without K cut into slices over workgroups whose slabs are added up afterwards."""
     g = torch.Generator().manual_seed(m * 3 + n)
     a = torch.randn(m, k, generator=g).bfloat16()
     if epi:
@@ -420,6 +420,10 @@ def test_gemm_bf16_panel_shapes(lib, m, n, k, epi):
         tol = 2e-5
     lib.gemm_bf16(a.to(DEV), w.to(DEV), out, epi)
     assert _rel(out, want) < tol
+    if not epi:
+        out16 = torch.full((m, n), float("nan"), device=DEV, dtype=torch.bfloat16)
+        lib.gemm_bf16(a.to(DEV), w.to(DEV), out16, epi)
+        assert _rel(out16, want) < 1e-2
 
 
 def test_attention_long_context(lib):
