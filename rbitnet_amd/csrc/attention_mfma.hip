@@ -306,8 +306,11 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
 //
 // With one split the result is written directly; with more, partial states go to the
 // workspace and attn_decode_combine_kernel adds them.  (Combining inside this kernel by a
-// ticket counter was tried: the device-scope fences it needs write back and invalidate the
-// L2 of every XCD and cost far more than the launch they save.)
+// ticket counter was tried twice.  With device-scope fences: they write back and invalidate
+// the L2 of every XCD and cost far more than the launch they save.  With fence-free
+// device-coherent stores, loads and a relaxed counter: correct, but the chain store
+// acknowledgement -> counter -> uncached loads takes as long as the second launch at 4
+// splits and much longer at 16 or more.)
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
   union {
