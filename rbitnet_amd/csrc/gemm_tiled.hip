@@ -1,0 +1,525 @@
+// Products with many tokens (prefill) and with 17..64 tokens: tiles of W and of the tokens
+// through LDS, MFMA 32x32x16 bf16, float32 accumulation.  W rows are the row operand of the
+// MFMA and the tokens its columns.
+//
+// Epilogue 1 expects W with gate and up rows interleaved in blocks of 16 and writes
+// silu(gate) * up (llama/model.rs:297-302 of the reference) instead of the two products.
+//
+// Reference loop: y[o] = sum_i W[i + o * n_in] * x[i]  (llama/model.rs:67-91).
+#include "api.h"
+#include "gemm_internal.h"
+
+// Adds up the [M, N] slabs of partial sums that the K slices of a product wrote, in slice
+// order (the same order whatever else runs), and converts to the output type.
+template <typename TO>
+__global__ void gemm_sum_slabs_kernel(const float* __restrict__ slabs, TO* __restrict__ c, int parts, size_t count) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float v = 0.f;
+  for (int p = 0; p < parts; ++p) v += slabs[(size_t)p * count + i];
+  Num<TO>::store(c + i, v);
+}
+
+// Which tile a workgroup computes.  Workgroup ids go round robin over the 8 XCDs, each with
+// an L2 of its own: every XCD gets a contiguous range of the tile order, and the order runs
+// through groups of TG_GROUP_M token tiles, all row tiles of a group before the next group.  The
+// 32 workgroups that an XCD runs at a time then cover about 8 x 4 tiles and walk K together,
+// so 12 tile rows come from beyond L2 per step for 32 tiles' worth of products.
+#define TG_GROUP_M 8
+__device__ __forceinline__ bool tile_of_workgroup(int m_tiles, int n_tiles, int* mt, int* nt) {
+  const int tiles = m_tiles * n_tiles;
+  const int per_xcd = (tiles + 7) / 8;
+  const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (t >= tiles) return false;
+  const int in_group = TG_GROUP_M * n_tiles;
+  const int first_m = t / in_group * TG_GROUP_M;
+  const int rows = min(m_tiles - first_m, TG_GROUP_M);
+  const int r = t % in_group;
+  *mt = first_m + r % rows;
+  *nt = r / rows;
+  return true;
+}
+
+#define TG_BK 64
+#define TG_LD 72          // bf16 elements per LDS row: 64 + 8 of padding, so that the 16 lanes
+                          // of a quarter wave read 16 different 16-byte bank groups
+
+template <int BN, int BM, int WN, int WM, int P, int EPI, bool KTAIL, typename TO>
+__global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
+                                                         const bf16_t* __restrict__ w, TO* __restrict__ c,
+                                                         int m, int n, int k, int m_tiles, int n_tiles) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int TN = WN / 32, TM = WM / 32;
+  constexpr int WAVES_N = BN / WN;
+  constexpr int NT = 64 * (BN / WN) * (BM / WM);      // threads: one wave per WN x WM piece of the tile
+  constexpr int W_CHUNKS = BN * 8 / NT, X_CHUNKS = BM * 8 / NT;
+  static_assert(BN * 8 % NT == 0 && BM * 8 % NT == 0 && NT % 8 == 0, "tile does not divide among the threads");
+  bf16_t* ws = reinterpret_cast<bf16_t*>(smem);                      // [2][BN][TG_LD]
+  bf16_t* xs = ws + 2 * BN * TG_LD;                                  // [2][BM][TG_LD]
+
+  int mt, nt;
+  if (!tile_of_workgroup(m_tiles, n_tiles, &mt, &nt)) return;
+  const int m0 = mt * BM;
+  const int n0 = nt * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wn0 = (wave % WAVES_N) * WN;
+  const int wm0 = (wave / WAVES_N) * WM;
+  const int l32 = lane & 31;
+  const int g = lane >> 5;
+
+  f32x16_t acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // ---- pipeline: tile kt is multiplied out of LDS while tiles kt + 1 .. kt + P - 1 are on
+  // their way from memory in registers (P - 1 tiles of latency hidden) and one of them is
+  // moved into the other LDS buffer.  Loads carry no conditions: rows beyond N or M are read
+  // from the last row and never stored, chunks beyond K are read from the last chunk and
+  // zeroed on their way into LDS.  (With conditions the compiler cannot count outstanding
+  // loads and waits for all of them.)
+  uint4 wreg[P][W_CHUNKS], xreg[P][X_CHUNKS];
+  // addresses: a 64-bit base per tile (the same for the whole workgroup) plus a 32-bit
+  // element offset per chunk; a tile spans at most 256 rows, so the offsets fit
+  const bf16_t* wtile = w + (size_t)n0 * k;
+  const bf16_t* xtile = x + (size_t)m0 * k;
+  uint32_t woff[W_CHUNKS], xoff[X_CHUNKS];
+#pragma unroll
+  for (int i = 0; i < W_CHUNKS; ++i) {
+    int row = (tid + NT * i) / 8;
+    if (n0 + row > n - 1) row = n - 1 - n0;
+    woff[i] = (uint32_t)row * (uint32_t)k;
+  }
+#pragma unroll
+  for (int i = 0; i < X_CHUNKS; ++i) {
+    int row = (tid + NT * i) / 8;
+    if (m0 + row > m - 1) row = m - 1 - m0;
+    xoff[i] = (uint32_t)row * (uint32_t)k;
+  }
+  const int kc = (tid % 8) * 8;             // this thread's chunk offset inside a tile (the same for all i)
+  auto load_global = [&](int slot, int kt) {
+    int col = kt * TG_BK + kc;
+    if (col > k - 8) col = k - 8;           // beyond K: any valid address; the data is zeroed in store_lds
+#pragma unroll
+    for (int i = 0; i < W_CHUNKS; ++i) wreg[slot][i] = load16(wtile + (woff[i] + (uint32_t)col));
+#pragma unroll
+    for (int i = 0; i < X_CHUNKS; ++i) xreg[slot][i] = load16(xtile + (xoff[i] + (uint32_t)col));
+  };
+  auto store_lds = [&](int slot, int kt) {
+    const int buf = kt & 1;
+    const bool in = !KTAIL || kt * TG_BK + kc < k;
+#pragma unroll
+    for (int i = 0; i < W_CHUNKS; ++i) {
+      const int q = tid + NT * i;
+      *reinterpret_cast<uint4*>(ws + ((size_t)buf * BN + q / 8) * TG_LD + kc) = in ? wreg[slot][i] : zero16();
+    }
+#pragma unroll
+    for (int i = 0; i < X_CHUNKS; ++i) {
+      const int q = tid + NT * i;
+      *reinterpret_cast<uint4*>(xs + ((size_t)buf * BM + q / 8) * TG_LD + kc) = in ? xreg[slot][i] : zero16();
+    }
+  };
+  auto multiply = [&](int kt) {
+    const bf16_t* wb = ws + (size_t)(kt & 1) * BN * TG_LD;
+    const bf16_t* xb = xs + (size_t)(kt & 1) * BM * TG_LD;
+    if (NT <= 256) {
+      // fragments of k-step ks + 1 are requested from LDS before the MFMAs of k-step ks
+      Frag8 a[2][TN], b[2][TM];
+      auto load_frags = [&](int buf2, int ks) {
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+          a[buf2][i].u = *reinterpret_cast<const uint4*>(wb + (size_t)(wn0 + 32 * i + l32) * TG_LD + ks * 16 + g * 8);
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+          b[buf2][j].u = *reinterpret_cast<const uint4*>(xb + (size_t)(wm0 + 32 * j + l32) * TG_LD + ks * 16 + g * 8);
+      };
+      load_frags(0, 0);
+#pragma unroll
+      for (int ks = 0; ks < TG_BK / 16; ++ks) {
+        if (ks + 1 < TG_BK / 16) load_frags((ks + 1) & 1, ks + 1);
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+          for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[ks & 1][i], b[ks & 1][j], acc[i][j]);
+      }
+    } else {
+      // 8 waves: two per SIMD cover each other's LDS latency, and registers are scarce
+#pragma unroll
+      for (int ks = 0; ks < TG_BK / 16; ++ks) {
+        Frag8 a[TN], b[TM];
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+          a[i].u = *reinterpret_cast<const uint4*>(wb + (size_t)(wn0 + 32 * i + l32) * TG_LD + ks * 16 + g * 8);
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+          b[j].u = *reinterpret_cast<const uint4*>(xb + (size_t)(wm0 + 32 * j + l32) * TG_LD + ks * 16 + g * 8);
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+          for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+      }
+    }
+  };
+
+  const int k_tiles = (k + TG_BK - 1) / TG_BK;
+  // tiles beyond the last are loaded as well (clamped) and never stored: the loop body stays
+  // free of conditions on loads
+#pragma unroll
+  for (int sl = 0; sl < P; ++sl) load_global(sl, sl);
+  store_lds(0, 0);
+  __syncthreads();
+  int kt = 0;
+  for (; kt + P <= k_tiles; kt += P) {        // P iterations per trip, so that the register slots are static
+#pragma unroll
+    for (int u = 0; u < P; ++u) {
+      // slot u held tile kt + u (now in LDS): reuse it for tile kt + u + P
+      load_global(u, kt + u + P);
+      multiply(kt + u);
+      if (kt + u + 1 < k_tiles) store_lds((u + 1) % P, kt + u + 1);
+      __syncthreads();
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < P; ++u) {               // the last k_tiles % P tiles
+    if (kt + u < k_tiles) {
+      multiply(kt + u);
+      if (kt + u + 1 < k_tiles) store_lds((u + 1) % P, kt + u + 1);
+      __syncthreads();
+    }
+  }
+
+  // ---- lane holds, per (i, j): token m0 + wm0 + 32 j + l32, W rows base + 8 (e / 4) + 4 g + e % 4
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int mm = m0 + wm0 + 32 * j + l32;
+      if (mm >= m) continue;
+      const int nbase = n0 + wn0 + 32 * i;
+      if (EPI == 0) {
+        TO* dst = c + (size_t)mm * n;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int nn = nbase + 8 * (e / 4) + 4 * g + (e % 4);
+          if (nn < n) Num<TO>::store(dst + nn, acc[i][j][e]);
+        }
+      } else {
+        const int half_n = n / 2;
+        TO* dst = c + (size_t)mm * half_n;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int nn = nbase / 2 + 8 * (e / 4) + 4 * g + (e % 4);
+          if (nn < half_n) Num<TO>::store(dst + nn, silu_f32(acc[i][j][e]) * acc[i][j][e + 8]);
+        }
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// The same product with the tiles brought from memory straight into LDS
+// (global_load_lds_dwordx4: no registers, no LDS store instruction), S stages deep.
+//
+// A wave's load instruction fills 1 KB of LDS in lane order, so rows cannot be padded.  Rows
+// of BK elements are kept dense and the 16-byte chunks of a row are permuted instead: chunk c
+// of row r lies in slot c ^ swz(r), swz(r) = (r / rows per 256 bytes) % chunks per row.  The
+// permutation is applied on the memory side (which chunk a lane fetches), and the 16 lanes of
+// a quarter wave that read one chunk column of 16 rows then hit 16 different bank groups.
+//
+// The loads are inline assembly, so the compiler neither counts nor waits for them: the
+// kernel waits itself (s_waitcnt vmcnt) for the stage it is about to read, leaving the
+// younger stages in flight.  There is no other memory access in the main loop.
+template <int N>
+__device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+__device__ __forceinline__ void load_to_lds16(const bf16_t* base, uint32_t byte_offset, uint32_t lds_byte_address) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds_byte_address), "v"(byte_offset), "s"(base)
+      : "memory");
+}
+
+template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO>
+__global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(const bf16_t* __restrict__ x,
+                                                       const bf16_t* __restrict__ w, TO* __restrict__ c,
+                                                       float* __restrict__ slabs, int m, int n, int k, int m_tiles,
+                                                       int n_tiles, int k_tiles) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  constexpr int TN = WN / 32, TM = WM / 32;
+  constexpr int WAVES_N = BN / WN;
+  constexpr int NWAVES = (BN / WN) * (BM / WM);
+  constexpr int CPR = BK / 8;                   // 16-byte chunks per row
+  constexpr int RPW = 64 / CPR;                 // rows one wave-wide load covers
+  constexpr int RPB = 128 / BK;                 // rows per 256 bytes of LDS
+  constexpr int W_LOADS = BN / RPW / NWAVES, X_LOADS = BM / RPW / NWAVES;
+  constexpr int LOADS = W_LOADS + X_LOADS;      // per thread and stage
+  constexpr int STAGE = (BN + BM) * BK;         // elements
+  static_assert(BN % (RPW * NWAVES) == 0 && BM % (RPW * NWAVES) == 0, "tile does not divide among the waves");
+  static_assert(S >= 2 && LOADS * (S - 1) < 64, "too many loads in flight for the counter");
+  bf16_t* lds = reinterpret_cast<bf16_t*>(smem);
+
+  int mt, nt;
+  if (!tile_of_workgroup(m_tiles, n_tiles, &mt, &nt)) return;
+  const int m0 = mt * BM;
+  const int n0 = nt * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn0 = (wave % WAVES_N) * WN;
+  const int wm0 = (wave / WAVES_N) * WM;
+  const int l32 = lane & 31;
+  const int g = lane >> 5;
+
+  f32x16_t acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // ---- what this lane fetches: wave-wide load q covers rows q * RPW .. + RPW - 1 of a tile
+  const bf16_t* wtile = w + (size_t)n0 * k;
+  const bf16_t* xtile = x + (size_t)m0 * k;
+  uint32_t woff[W_LOADS], xoff[X_LOADS];        // byte offsets from the tile's first element, without the k-tile
+#pragma unroll
+  for (int i = 0; i < W_LOADS; ++i) {
+    const int row = (wave + NWAVES * i) * RPW + lane / CPR;
+    const int chunk = (lane % CPR) ^ ((row / RPB) % CPR);
+    int grow = row;
+    if (n0 + grow > n - 1) grow = n - 1 - n0;   // rows beyond N: any valid row, never stored
+    woff[i] = ((uint32_t)grow * (uint32_t)k + chunk * 8) * 2u;
+  }
+#pragma unroll
+  for (int i = 0; i < X_LOADS; ++i) {
+    const int row = (wave + NWAVES * i) * RPW + lane / CPR;
+    const int chunk = (lane % CPR) ^ ((row / RPB) % CPR);
+    int grow = row;
+    if (m0 + grow > m - 1) grow = m - 1 - m0;
+    xoff[i] = ((uint32_t)grow * (uint32_t)k + chunk * 8) * 2u;
+  }
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;      // LDS byte address of stage 0
+  const int kt0 = blockIdx.y * k_tiles;                    // this workgroup's slice of K: k_tiles tiles from here
+  auto issue = [&](int kt) {
+    const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
+    const uint32_t kbytes = (uint32_t)(kt0 + kt) * (BK * 2);
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i)
+      load_to_lds16(wtile, woff[i] + kbytes, stage + (uint32_t)(wave + NWAVES * i) * 1024u);
+#pragma unroll
+    for (int i = 0; i < X_LOADS; ++i)
+      load_to_lds16(xtile, xoff[i] + kbytes, stage + (uint32_t)(BN * BK * 2) + (uint32_t)(wave + NWAVES * i) * 1024u);
+  };
+
+  // ---- fragments: row base + 32 i + l32, chunk 2 ks + g, found in slot chunk ^ swz(l32)
+  const int sw = (l32 / RPB) % CPR;
+  const bf16_t* wfrag = lds + (size_t)(wn0 + l32) * BK;
+  const bf16_t* xfrag = lds + (size_t)BN * BK + (size_t)(wm0 + l32) * BK;
+  auto multiply = [&](int kt) {
+    const bf16_t* wb = wfrag + (size_t)(kt % S) * STAGE;
+    const bf16_t* xb = xfrag + (size_t)(kt % S) * STAGE;
+    Frag8 a[2][TN], b[2][TM];
+    auto load_frags = [&](int buf2, int ks) {
+      const int slot = ((2 * ks + g) ^ sw) * 8;
+#pragma unroll
+      for (int i = 0; i < TN; ++i) a[buf2][i].u = *reinterpret_cast<const uint4*>(wb + 32 * i * BK + slot);
+#pragma unroll
+      for (int j = 0; j < TM; ++j) b[buf2][j].u = *reinterpret_cast<const uint4*>(xb + 32 * j * BK + slot);
+    };
+    load_frags(0, 0);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      if (ks + 1 < BK / 16) load_frags((ks + 1) & 1, ks + 1);
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[ks & 1][i], b[ks & 1][j], acc[i][j]);
+    }
+  };
+
+#pragma unroll
+  for (int s = 0; s < S - 1; ++s)
+    if (s < k_tiles) issue(s);
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    // tile kt must have landed; in the steady state the S - 2 tiles after it stay in flight
+    if (kt + S - 2 < k_tiles) wait_vm<LOADS * (S - 2)>();
+    else wait_vm<0>();
+    __syncthreads();                  // everyone's part of tile kt is in LDS, and tile kt - 1 has been read by all
+    if (kt + S - 1 < k_tiles) issue(kt + S - 1);      // into the stage tile kt - 1 occupied
+    multiply(kt);
+  }
+
+  // ---- lane holds, per (i, j): token m0 + wm0 + 32 j + l32, W rows base + 8 (e / 4) + 4 g + e % 4
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int mm = m0 + wm0 + 32 * j + l32;
+      if (mm >= m) continue;
+      const int nbase = n0 + wn0 + 32 * i;
+      if (EPI == 0) {
+        // a slice of K: partial sums go to this slice's [M, N] slab, to be added up in a fixed order
+        float* slab = slabs ? slabs + ((size_t)blockIdx.y * m + mm) * n : nullptr;
+        TO* dst = c + (size_t)mm * n;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int nn = nbase + 8 * (e / 4) + 4 * g + (e % 4);
+          if (nn >= n) continue;
+          if (slab) slab[nn] = acc[i][j][e];
+          else Num<TO>::store(dst + nn, acc[i][j][e]);
+        }
+      } else {
+        const int half_n = n / 2;
+        TO* dst = c + (size_t)mm * half_n;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int nn = nbase / 2 + 8 * (e / 4) + 4 * g + (e % 4);
+          if (nn < half_n) Num<TO>::store(dst + nn, silu_f32(acc[i][j][e]) * acc[i][j][e + 8]);
+        }
+      }
+    }
+}
+
+template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO>
+static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s,
+                          int parts = 1, float* slabs = nullptr) {
+  const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
+  RB_REQUIRE(parts >= 1 && (k / BK) % parts == 0 && (parts == 1 || (slabs && EPI == 0)),
+             "rb_gemm_bf16: internal: bad K split %d", parts);
+  const long long tiles = (long long)m_tiles * n_tiles;
+  RB_REQUIRE(tiles < (1LL << 30), "rb_gemm_bf16: too many tiles");
+  RB_REQUIRE(k % BK == 0, "rb_gemm_bf16: the direct-to-LDS kernel needs K=%d to be a multiple of %d", k, BK);
+  // byte offsets inside a tile are 32-bit
+  RB_REQUIRE((long long)(BN > BM ? BN : BM) * k * 2 < (1LL << 32), "rb_gemm_bf16: K=%d too long for this kernel", k);
+  const size_t lds = (size_t)S * (BN + BM) * BK * sizeof(bf16_t);
+  auto kern = gemm_dma_kernel<BN, BM, WN, WM, BK, S, EPI, TO>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    RB_REQUIRE(e == hipSuccess, "rb_gemm_bf16: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    configured = true;
+  }
+  const dim3 grid((unsigned)((tiles + 7) / 8 * 8), (unsigned)parts);
+  kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, parts > 1 ? slabs : nullptr, m, n, k, m_tiles,
+                                                      n_tiles, k / BK / parts);
+  if (parts > 1) {
+    const size_t count = (size_t)m * n;
+    gemm_sum_slabs_kernel<TO><<<(unsigned)((count + 255) / 256), 256, 0, s>>>(slabs, (TO*)c, parts, count);
+  }
+  return 0;
+}
+
+// ------------------------------------------------------------------ 17 .. 64 tokens, K % 64 == 0
+// The same kernel with one token tile: W streams through LDS three stages deep, two
+// workgroups per compute unit.  Few rows of W: K is also cut into slices over workgroups
+// (grid.y); each slice writes its partial sums to its own [M, N] slab of a workspace, and
+// gemm_sum_slabs_kernel adds them up in a fixed order.
+static int g_stream_parts = 0;
+extern "C" void rb_tune_stream_parts(int parts) { g_stream_parts = parts; }      // experiments only; 0 = built-in
+
+static int stream_parts(int m, int n, int k, int epilogue) {
+  if (m <= 16 || m > 64 || k % 64 != 0 || (long long)k * 256 >= (1LL << 32)) return 0;      // not for this kernel
+  if (epilogue == 1) return 1;
+  const int tiles = (n + 127) / 128;
+  const int kt = k / 64;
+  if (g_stream_parts && kt % g_stream_parts == 0) return g_stream_parts;
+  // every slice writes and re-reads an [M, N] slab (8 bytes per element): keep that under half
+  // of W's bytes, the slices at 16 and at least 4 tiles deep, the workgroups at one per compute
+  // unit (more slices cost more in slabs than they gain: measured on N = 4096 and 6144)
+  int cap = k / (8 * m);
+  if (cap > 16) cap = 16;
+  int best = 1;
+  for (int p = 1; p <= cap; ++p) {
+    if (kt % p != 0 || kt / p < 4) continue;
+    if ((long long)tiles * p <= 256) best = p;
+  }
+  return best;
+}
+
+template <int EPI, typename TO>
+static int launch_stream(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int m, int n, int k,
+                         hipStream_t s) {
+  const int parts = stream_parts(m, n, k, EPI);
+  RB_REQUIRE(parts >= 1, "rb_gemm_bf16: internal: not a product for the streaming kernel");
+  RB_REQUIRE(parts == 1 || workspace != nullptr, "rb_gemm_bf16: M=%d N=%d K=%d needs a workspace of %lld floats", m, n,
+             k, (long long)parts * m * n);
+  return launch_dma_cfg<128, 64, 32, 64, 64, 3, EPI, TO>(x, w, c, m, n, k, s, parts, workspace);
+}
+
+static int g_tile_cfg = 0;
+extern "C" void rb_tune_tiles(int cfg) { g_tile_cfg = cfg; }      // experiments only; 0 = built-in choice
+
+template <int BN, int BM, int WN, int WM, int P, int EPI, typename TO>
+static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
+  const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
+  const long long tiles = (long long)m_tiles * n_tiles;
+  RB_REQUIRE(tiles < (1LL << 30), "rb_gemm_bf16: too many tiles");
+  const size_t lds = (size_t)2 * (BN + BM) * TG_LD * sizeof(bf16_t);
+  const bool tail = k % TG_BK != 0;
+  auto kern = tail ? gemm_tiled_kernel<BN, BM, WN, WM, P, EPI, true, TO>
+                   : gemm_tiled_kernel<BN, BM, WN, WM, P, EPI, false, TO>;
+  static bool configured[2] = {false, false};
+  if (!configured[tail]) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    RB_REQUIRE(e == hipSuccess, "rb_gemm_bf16: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    configured[tail] = true;
+  }
+  const int grid = (int)((tiles + 7) / 8 * 8);
+  kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, m, n, k, m_tiles, n_tiles);
+  return 0;
+}
+
+// Which tile for which product.  Measured on the Llama-3-8B products at M = 2048 .. 8192: the
+// kernels are bound by what they pull from L2 and LDS (a 128 x 128 x 64 tile needs a byte per
+// 64 flop, a 256 x 256 one half of that), so the largest tile that still gives every compute
+// unit work wins: 256 x 256 when there are at least ~160 such tiles, else 128 x 128 (two
+// workgroups per compute unit).  The direct-to-LDS kernel is 10-20 % faster than the one that
+// stages tiles in registers and is used whenever K is a multiple of its 64-deep tile.
+template <int EPI, typename TO>
+static int launch_tiled(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
+  int cfg = g_tile_cfg;
+  if (cfg == 0) {
+    const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
+    const long long t256x128 = (long long)((m + 127) / 128) * ((n + 255) / 256);
+    const bool dma = k % 64 == 0 && (long long)k * 512 < (1LL << 32);
+    if (dma) cfg = t256 >= 160 ? 4 : 5;
+    else if (t256 >= 160) cfg = 3;
+    else if (k >= 8192 && t256x128 >= 200) cfg = 2;
+    else cfg = 1;
+  }
+  switch (cfg) {
+    case 5: return launch_dma_cfg<128, 128, 64, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+    case 4: return launch_dma_cfg<256, 256, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+    case 3: return launch_tiled_cfg<256, 256, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+    case 2: return launch_tiled_cfg<256, 128, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+    default: return launch_tiled_cfg<128, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+  }
+}
+
+
+#define RB_BY_OUTPUT(FN, ...)                                                              \
+  (epilogue == 0 ? (dtype_out == RB_F32 ? FN<0, float>(__VA_ARGS__) : FN<0, bf16_t>(__VA_ARGS__)) \
+                 : (dtype_out == RB_F32 ? FN<1, float>(__VA_ARGS__) : FN<1, bf16_t>(__VA_ARGS__)))
+
+int gemm_tiled_launch(const bf16_t* x, const bf16_t* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
+                      hipStream_t s) {
+  return RB_BY_OUTPUT(launch_tiled, x, w, c, m, n, k, s);
+}
+
+int gemm_stream_parts(int m, int n, int k, int epilogue) { return stream_parts(m, n, k, epilogue); }
+
+int gemm_stream_launch(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int dtype_out, int epilogue,
+                       int m, int n, int k, hipStream_t s) {
+  return RB_BY_OUTPUT(launch_stream, x, w, c, workspace, m, n, k, s);
+}
