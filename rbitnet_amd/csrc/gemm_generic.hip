@@ -65,11 +65,84 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TI* __restrict_
   }
 }
 
+// Float32 operands and at most 16 tokens (the float32 path's decode step): bound by reading W
+// once.  A wave owns 4 rows of W and walks all of K with 16-byte loads (a row is read as
+// 1 KB contiguous per instruction); the tokens' 1024-deep chunk goes through LDS once for
+// the 4 waves; every lane keeps a partial sum per (row, token) and the wave adds them up at
+// the end.  K must be a multiple of 4.
+#define GS_ROWS 4
+#define GS_KC 1024
+
+template <int MT>
+__global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __restrict__ a, const float* __restrict__ w,
+                                                              float* __restrict__ c, int m, int n, int k) {
+  __shared__ float4 xs[MT][GS_KC / 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int row0 = (blockIdx.x * 4 + wave) * GS_ROWS;
+  float acc[GS_ROWS][MT];
+#pragma unroll
+  for (int r = 0; r < GS_ROWS; ++r)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[r][t] = 0.f;
+  const float* wrow[GS_ROWS];
+#pragma unroll
+  for (int r = 0; r < GS_ROWS; ++r) wrow[r] = w + (size_t)(row0 + r < n ? row0 + r : n - 1) * k;
+
+  for (int k0 = 0; k0 < k; k0 += GS_KC) {
+    __syncthreads();                  // the previous chunk has been used by every wave
+    for (int idx = tid; idx < MT * (GS_KC / 4); idx += 256) {
+      const int t = idx / (GS_KC / 4), q = idx % (GS_KC / 4);
+      const int kk = k0 + 4 * q;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (t < m && kk < k) v = *reinterpret_cast<const float4*>(a + (size_t)t * k + kk);
+      xs[t][q] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int step = 0; step < GS_KC / 256; ++step) {
+      const int q = step * 64 + lane;
+      const int kk = k0 + 4 * q;
+      const int kl = kk < k ? kk : k - 4;            // beyond K: a valid address; the tokens' chunk holds zeros there
+      float4 wv[GS_ROWS];
+#pragma unroll
+      for (int r = 0; r < GS_ROWS; ++r) wv[r] = *reinterpret_cast<const float4*>(wrow[r] + kl);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const float4 xv = xs[t][q];
+#pragma unroll
+        for (int r = 0; r < GS_ROWS; ++r) {
+          acc[r][t] = fmaf(wv[r].x, xv.x, acc[r][t]);
+          acc[r][t] = fmaf(wv[r].y, xv.y, acc[r][t]);
+          acc[r][t] = fmaf(wv[r].z, xv.z, acc[r][t]);
+          acc[r][t] = fmaf(wv[r].w, xv.w, acc[r][t]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < GS_ROWS; ++r)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const float v = wave_sum(acc[r][t]);
+      if (lane == 0 && row0 + r < n && t < m) c[(size_t)t * n + row0 + r] = v;
+    }
+}
+
 extern "C" int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dtype_out, int m, int n,
                                int k, void* stream) {
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_generic: bad sizes M=%d N=%d K=%d", m, n, k);
   if (m == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  if (dtype_in == RB_F32 && dtype_out == RB_F32 && m <= 16 && k % 4 == 0) {
+    const unsigned blocks = (unsigned)((n + 4 * GS_ROWS - 1) / (4 * GS_ROWS));
+    const float* af = (const float*)a;
+    const float* wf = (const float*)w;
+    if (m <= 4) gemm_f32_skinny_kernel<4><<<blocks, 256, 0, s>>>(af, wf, (float*)c, m, n, k);
+    else if (m <= 8) gemm_f32_skinny_kernel<8><<<blocks, 256, 0, s>>>(af, wf, (float*)c, m, n, k);
+    else gemm_f32_skinny_kernel<16><<<blocks, 256, 0, s>>>(af, wf, (float*)c, m, n, k);
+    RB_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid((n + GT - 1) / GT, (m + GT - 1) / GT);
   RB_REQUIRE(grid.y <= 65535, "rb_gemm_generic: M=%d too large for one launch", m);
   if (dtype_in == RB_F32 && dtype_out == RB_F32)

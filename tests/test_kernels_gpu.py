@@ -44,7 +44,8 @@ def test_reference_matvec_vectors(lib):
     assert torch.allclose(c.cpu(), torch.tensor([[1.75, 0.75, -1.5]]), atol=1e-5)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 130, 67), (65, 64, 16), (130, 200, 333)])
+@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 130, 67), (65, 64, 16), (130, 200, 333), (1, 130, 64), (8, 1000, 2052),
+                                   (16, 33, 4096), (5, 300, 1028), (4, 17, 4), (17, 50, 64)])
 def test_gemm_generic_f32(lib, m, n, k):
     g = torch.Generator().manual_seed(m * 1000 + n)
     a = torch.randn(m, k, generator=g)
