@@ -569,6 +569,251 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// The same decode step on the matrix cores, for any number of query heads per kv head up to
+// 16: scores S^T[key, head] = K q^T and outputs O^T[d, head] = V^T P^T as 16x16x32 MFMAs with
+// the heads as the 16 columns (columns beyond the group are zero queries).  The vector
+// kernel above spends 8 dot products and 8 multiply-adds per key element at 8 heads per kv
+// head and is bound by that arithmetic; here the work per key does not grow with the group.
+//
+// A wave takes a page at a time.  K rows go from memory straight into MFMA operands.  The
+// second product needs V^T (8 keys of one d per lane): the page of V is brought into the
+// wave's own LDS area by direct loads (dense 256- or 128-byte rows, 16-byte chunks permuted
+// by (key / 4) % 4 so that the four lane groups of a transposed read hit different banks)
+// and read back as 16-bit values.  The probabilities leave the first MFMA as 4 keys per lane
+// and tile; the k index of the second product is ordered so that a lane's own 8 values
+// (keys 4 grp + 0..3 of two tiles) are its operand, and V^T is read in the same order.
+// Rows of the last page beyond the position may hold anything (0 x NaN would spoil the
+// product): they are cleared in LDS, and the token's own row is put there (FUSED).
+template <int D, bool FUSED>
+__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
+    const float* __restrict__ qkv, const bf16_t* __restrict__ q_in, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int style, bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out,
+    const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
+    int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws) {
+  constexpr int KS = D / 32;          // depth steps of the score product
+  constexpr int DT = D / 16;          // d tiles of the output product
+  constexpr int HALF = D / 2;
+  constexpr int CPR = D / 8;          // 16-byte chunks per row of V
+  constexpr int RPI = 64 / CPR;       // rows one direct load instruction covers
+  constexpr int VI = RB_PAGE / RPI;   // direct load instructions per page
+  constexpr int DL = D / 64;          // elements of a row per lane
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  uint16_t* vpages = reinterpret_cast<uint16_t*>(smem);                    // [4 waves][64 keys][D]
+  uint16_t* q_h = vpages + 4 * RB_PAGE * D;                                // [16][D]
+  uint16_t* knew_h = q_h + 16 * D;
+  uint16_t* vnew_h = knew_h + D;
+  float* red_m = reinterpret_cast<float*>(vnew_h + D);                     // [4][16]
+  float* red_l = red_m + 64;                                               // [4][64]
+  float* red_acc = reinterpret_cast<float*>(smem);                         // [4][16][D], over the pages at the end
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // the same for the whole wave: LDS addresses go to a scalar register
+  const int c16 = lane & 15, grp = lane >> 4;
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int G = n_heads / n_kv;
+  const int pos = tok_pos[b];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first_page = lo / RB_PAGE, last_page = pos / RB_PAGE;
+  const int32_t* pages = block_table + (size_t)b * bt_stride;
+
+  // ---- q of the group (rotated here when FUSED) as bfloat16 rows in LDS, zero rows beyond it
+  if (FUSED) {
+    const int row_width = (n_heads + 2 * n_kv) * D;
+    const float* src = qkv + (size_t)b * row_width;
+    const float* cr = cos_t ? cos_t + (size_t)pos * HALF : nullptr;
+    const float* sr = cos_t ? sin_t + (size_t)pos * HALF : nullptr;
+    for (int idx = tid; idx < 17 * HALF; idx += 256) {
+      const int gg = idx / HALF, i = idx - gg * HALF;
+      const int i0 = style == 0 ? 2 * i : i, i1 = style == 0 ? 2 * i + 1 : i + HALF;
+      uint16_t* dst = gg < 16 ? q_h + gg * D : knew_h;
+      if (gg < 16 && gg >= G) {
+        dst[i0] = 0;
+        dst[i1] = 0;
+        continue;
+      }
+      const float* h = gg < 16 ? src + (size_t)(kvh * G + gg) * D : src + (size_t)(n_heads + kvh) * D;
+      const float x0 = h[i0], x1 = h[i1];
+      float y0 = x0, y1 = x1;
+      if (cr) {
+        const float c = cr[i], sn = sr[i];
+        y0 = x0 * c - x1 * sn;
+        y1 = x0 * sn + x1 * c;
+      }
+      dst[i0] = f32_to_bf16_bits(y0);
+      dst[i1] = f32_to_bf16_bits(y1);
+    }
+    for (int d = tid; d < D; d += 256) vnew_h[d] = f32_to_bf16_bits(src[(size_t)(n_heads + n_kv + kvh) * D + d]);
+  } else {
+    for (int idx = tid; idx < 16 * D; idx += 256) {
+      const int gg = idx / D, d = idx - gg * D;
+      q_h[idx] = gg < G ? q_in[((size_t)b * n_heads + kvh * G + gg) * D + d].bits : (uint16_t)0;
+    }
+  }
+  __syncthreads();
+  if (FUSED && split == (last_page - first_page) % n_splits) {      // this workgroup owns the last page
+    const int page = pages[last_page];
+    const size_t at = ((size_t)page * n_kv + kvh) * RB_PAGE * D + (size_t)(pos % RB_PAGE) * D;
+    for (int d = tid; d < D; d += 256) {
+      k_pages[at + d].bits = knew_h[d];
+      v_pages[at + d].bits = vnew_h[d];
+    }
+  }
+  Frag8 qf[KS];
+#pragma unroll
+  for (int st = 0; st < KS; ++st) qf[st].u = *reinterpret_cast<const uint4*>(q_h + c16 * D + 32 * st + 8 * grp);
+
+  float m_run = -INFINITY, l_part = 0.f;
+  f32x4_t acc_o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) acc_o[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  uint16_t* vpage = vpages + wave * RB_PAGE * D;
+  const uint32_t vpage_lds = (uint32_t)(uintptr_t)vpage;
+
+  for (int pg = first_page + split + n_splits * wave; pg <= last_page; pg += 4 * n_splits) {
+    const int page = __builtin_amdgcn_readfirstlane(pages[pg]);
+    const size_t base = ((size_t)page * n_kv + kvh) * RB_PAGE * D;
+    // the reads of the previous page have all returned before its area is overwritten
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < VI; ++i) {
+      const int key = i * RPI + lane / CPR;
+      const int chunk = (lane % CPR) ^ ((key >> 2) & 3);
+      load_to_lds16(v_pages + base, (uint32_t)(key * D + chunk * 8) * 2u, vpage_lds + i * 1024u);
+    }
+    Frag8 kf[4][KS];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int st = 0; st < KS; ++st) kf[t][st].u = load16(k_pages + base + (size_t)(16 * t + c16) * D + 32 * st + 8 * grp);
+    if (FUSED && pg == last_page) {
+      // the token's own key is not in the cache yet (or only just): take it from LDS
+      const int t_new = (pos % RB_PAGE) / 16, r_new = pos % 16;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int st = 0; st < KS; ++st)
+          if (t == t_new && c16 == r_new) kf[t][st].u = *reinterpret_cast<const uint4*>(knew_h + 32 * st + 8 * grp);
+    }
+    // ---- scores: lane holds keys 16 t + 4 grp + i of head c16
+    f32x4_t sc[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      sc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int st = 0; st < KS; ++st) sc[t] = mfma16(kf[t][st], qf[st], sc[t]);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = pg * RB_PAGE + 16 * t + 4 * grp + i;
+        const float v = (key >= lo && key <= pos) ? sc[t][i] * scale_log2 : -INFINITY;
+        sc[t][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = __builtin_amdgcn_exp2f(sc[t][i] - m_safe);
+        sc[t][i] = pv;
+        psum += pv;
+      }
+    l_part = l_part * corr + psum;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc_o[dt][i] *= corr;
+    Frag8 pf[2];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      pf[s2].u.x = pack_bf16x2(sc[2 * s2][0], sc[2 * s2][1]);
+      pf[s2].u.y = pack_bf16x2(sc[2 * s2][2], sc[2 * s2][3]);
+      pf[s2].u.z = pack_bf16x2(sc[2 * s2 + 1][0], sc[2 * s2 + 1][1]);
+      pf[s2].u.w = pack_bf16x2(sc[2 * s2 + 1][2], sc[2 * s2 + 1][3]);
+    }
+    // ---- the page of V has arrived (loads complete in issue order, and K came after it)
+    wait_vm<0>();
+    if (pg == last_page) {
+      const int r_pos = pos % RB_PAGE;
+      for (int row = FUSED ? r_pos : r_pos + 1; row < RB_PAGE; ++row) {
+        const int d = lane * DL;
+        uint16_t* dst = vpage + row * D + (((d >> 3) ^ ((row >> 2) & 3)) * 8 + (d & 7));
+        const bool own = FUSED && row == r_pos;
+        if (DL == 2)
+          *reinterpret_cast<uint32_t*>(dst) = own ? *reinterpret_cast<const uint32_t*>(vnew_h + d) : 0u;
+        else
+          *dst = own ? vnew_h[d] : (uint16_t)0;
+      }
+    }
+    // ---- O^T[d, head] += V^T P^T: lane reads, for d = 16 dt + c16, the 8 keys of its group
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int d = 16 * dt + c16;
+      const uint16_t* col = vpage + (size_t)(4 * grp) * D + (((d >> 3) ^ grp) * 8 + (d & 7));
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        uint32_t wv[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          // pairs (e = 0, 1 of tile 2 s2; e = 2, 3: of tile 2 s2 + 1): keys 32 s2 + 16 (e / 2) + 4 grp + 2 (e % 2) + 0, 1
+          const int key0 = 32 * s2 + 16 * (e / 2) + 2 * (e % 2);
+          wv[e] = (uint32_t)col[(size_t)key0 * D] | ((uint32_t)col[(size_t)(key0 + 1) * D] << 16);
+        }
+        Frag8 vf;
+        vf.u = make_uint4(wv[0], wv[1], wv[2], wv[3]);
+        acc_o[dt] = mfma16(vf, pf[s2], acc_o[dt]);
+      }
+    }
+  }
+
+  // ---- the four waves' states into one (the pages' area is reused for the outputs)
+  __syncthreads();
+  if (c16 < G) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red_acc[((size_t)wave * 16 + c16) * D + 16 * dt + 4 * grp + i] = acc_o[dt][i];
+  }
+  red_l[wave * 64 + lane] = l_part;
+  if (grp == 0) red_m[wave * 16 + c16] = m_run;
+  __syncthreads();
+  for (int idx = tid; idx < G * D; idx += 256) {
+    const int gg = idx / D, d = idx % D;
+    float mx = red_m[gg];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) mx = fmaxf(mx, red_m[w * 16 + gg]);
+    const float m_safe = (mx == -INFINITY) ? 0.f : mx;
+    float a = 0.f, l = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = exp2f(red_m[w * 16 + gg] - m_safe);
+      a += red_acc[((size_t)w * 16 + gg) * D + d] * f;
+      const float* lw = red_l + w * 64 + gg;
+      l += ((lw[0] + lw[16]) + (lw[32] + lw[48])) * f;
+    }
+    if (n_splits == 1) {
+      out[((size_t)b * n_heads + kvh * G + gg) * D + d] = f32_to_bf16(l > 0.f ? a / l : 0.f);
+    } else {
+      float* dst = ws + (((size_t)b * n_heads + kvh * G + gg) * n_splits + split) * (D + 2);
+      dst[d] = a;
+      if (d == 0) {
+        dst[D] = mx;
+        dst[D + 1] = l;
+      }
+    }
+  }
+}
+
 template <int D>
 __global__ void attn_decode_combine_kernel(const float* __restrict__ ws, bf16_t* __restrict__ out, int n_splits) {
   const size_t row = blockIdx.x;            // sequence * heads + head
@@ -612,6 +857,31 @@ static void launch_decode(const DecodeArgs& a, hipStream_t s) {
   if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits);
 }
 
+template <int D, bool FUSED>
+static int launch_decode_mfma(const DecodeArgs& a, hipStream_t s) {
+  const size_t lds = (size_t)4 * RB_PAGE * D * 2 + 16 * D * 2 + 2 * D * 2 + (64 + 256) * sizeof(float);
+  auto kern = attn_decode_mfma_kernel<D, FUSED>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    RB_REQUIRE(e == hipSuccess, "decode attention: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    configured = true;
+  }
+  dim3 grid(a.n_splits, a.n_kv, a.n_seqs);
+  kern<<<grid, 256, lds, s>>>(a.qkv, a.q, a.cos_t, a.sin_t, a.style, a.k, a.v, a.out, a.tok_pos, a.bt, a.bt_stride,
+                              a.n_heads, a.n_kv, a.sl2, a.window, a.n_splits, a.ws);
+  if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits);
+  return 0;
+}
+
+// Which decode kernel: 0 = by group size (matrix cores from 2 query heads per kv head on: the
+// vector kernel's arithmetic grows with the group, and it is built for groups of 1, 2, 4 and 8
+// only; with one head per kv head the two are equally fast), 1 = always the matrix-core
+// kernel, 2 = never.  Experiments and tests only.
+static int g_decode_mfma = 0;
+extern "C" void rb_tune_decode_mfma(int mode) { g_decode_mfma = mode; }
+
 template <bool FUSED>
 static int dispatch_decode(const DecodeArgs& a, int head_dim, hipStream_t s, const char* who) {
   RB_REQUIRE(a.n_seqs > 0, "%s: empty batch", who);
@@ -624,8 +894,16 @@ static int dispatch_decode(const DecodeArgs& a, int head_dim, hipStream_t s, con
   RB_REQUIRE(a.window >= 0, "%s: negative window", who);
   RB_REQUIRE(a.n_splits == 1 || a.ws != nullptr, "%s: splits need a workspace", who);
   const int group = a.n_heads / a.n_kv;
-  RB_REQUIRE(group == 1 || group == 2 || group == 4 || group == 8,
-             "%s: %d query heads per kv head not supported (1, 2, 4, 8; use rb_attention_generic)", who, group);
+  const bool vector_ok = group == 1 || group == 2 || group == 4 || group == 8;
+  RB_REQUIRE(group <= 16, "%s: %d query heads per kv head not supported (at most 16; use rb_attention_generic)", who,
+             group);
+  RB_REQUIRE(g_decode_mfma != 2 || vector_ok, "%s: the vector kernel is built for 1, 2, 4 or 8 heads per kv head", who);
+  if (g_decode_mfma == 1 || !vector_ok || (g_decode_mfma == 0 && group > 1)) {
+    const int rc = head_dim == 128 ? launch_decode_mfma<128, FUSED>(a, s) : launch_decode_mfma<64, FUSED>(a, s);
+    if (rc) return rc;
+    RB_LAUNCH_CHECK();
+    return 0;
+  }
   if (head_dim == 128) {
     if (group == 1) launch_decode<128, 1, FUSED>(a, s);
     else if (group == 2) launch_decode<128, 2, FUSED>(a, s);

@@ -234,19 +234,6 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_tiled_kernel(
 // The loads are inline assembly, so the compiler neither counts nor waits for them: the
 // kernel waits itself (s_waitcnt vmcnt) for the stage it is about to read, leaving the
 // younger stages in flight.  There is no other memory access in the main loop.
-template <int N>
-__device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-
-__device__ __forceinline__ void load_to_lds16(const bf16_t* base, uint32_t byte_offset, uint32_t lds_byte_address) {
-  asm volatile(
-      "s_mov_b32 m0, %0\n\t"
-      "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %1, %2"
-      :
-      : "s"(lds_byte_address), "v"(byte_offset), "s"(base)
-      : "memory");
-}
-
 template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO>
 __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(const bf16_t* __restrict__ x,
                                                        const bf16_t* __restrict__ w, TO* __restrict__ c,

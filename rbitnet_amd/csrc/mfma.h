@@ -33,3 +33,21 @@ __device__ __forceinline__ uint4 load16(const void* p) { return *reinterpret_cas
 __device__ __forceinline__ uint4 zero16() { return make_uint4(0u, 0u, 0u, 0u); }
 
 __device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + expf(-v)); }
+
+// ---- memory -> LDS without registers (global_load_lds_dwordx4): the 64 lanes of a wave fetch
+// 16 bytes each from base + their byte offset, and the 1 KB lands at the given LDS address in
+// lane order.  The instruction is inline assembly, so the compiler neither counts nor waits
+// for it: wait with wait_vm<N>() (at most N vector memory operations of this wave still
+// outstanding; they complete in issue order) before the data is read from LDS.
+template <int N>
+__device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+__device__ __forceinline__ void load_to_lds16(const bf16_t* base, uint32_t byte_offset, uint32_t lds_byte_address) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds_byte_address), "v"(byte_offset), "s"(base)
+      : "memory");
+}

@@ -13,15 +13,26 @@ import numpy as np
 import torch
 
 
-def decode_splits(n_seqs: int, n_kv_heads: int) -> int:
+def split_bucket(max_kv_len: int) -> int:
+    """1, 2, 4, 8 or 16 by the longest context of the batch: about eight pages of 64 keys per
+    split (a workgroup walks four pages at a time; a page costs far less than the second
+    launch that combines splits, so short contexts are not split at all)."""
+    pages = (max(1, int(max_kv_len)) + 63) // 64
+    bucket = 1
+    while bucket < 16 and bucket * 2 <= pages // 8:
+        bucket *= 2
+    return bucket
+
+
+def decode_splits(n_seqs: int, n_kv_heads: int, bucket: int = 16) -> int:
     """Into how many workgroups the pages of one (sequence, kv head) are dealt in decode
-    attention: enough to give every compute unit about one workgroup, no more (each
-    workgroup already walks four pages at a time, and every split adds to the combination)."""
+    attention: what the context length asks for (`split_bucket`), but no more than gives
+    every compute unit about one workgroup (every split adds to the combination)."""
     import os
     forced = os.environ.get("RBITNET_DECODE_SPLITS")
     if forced:
         return max(1, int(forced))
-    return max(1, min(16, 256 // max(1, n_seqs * max(1, n_kv_heads))))
+    return max(1, min(int(bucket), 16, 256 // max(1, n_seqs * max(1, n_kv_heads))))
 
 
 class StepContext:
@@ -81,7 +92,7 @@ class StepContext:
         GPU, whatever the context length (each split strides over the pages)."""
         key = (n_heads, head_dim, n_kv_heads)
         if key not in self._workspaces:
-            n_splits = decode_splits(self.n_seqs, n_kv_heads)
+            n_splits = decode_splits(self.n_seqs, n_kv_heads, split_bucket(self.max_kv_len))
             ws = torch.empty(self.n_seqs * n_heads * n_splits * (head_dim + 2), dtype=torch.float32,
                              device=self.device)
             self._workspaces[key] = (n_splits, ws)

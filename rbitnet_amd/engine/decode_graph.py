@@ -25,9 +25,10 @@ class _StaticContext:
     """Has the attributes of `StepContext`, but every device tensor is a fixed view into
     one buffer that `DecodeGraph.run` refreshes before each replay."""
 
-    def __init__(self, device, n_seqs: int, group_keys: Sequence[int], table_width: int):
+    def __init__(self, device, n_seqs: int, group_keys: Sequence[int], table_width: int, bucket: int = 16):
         b = n_seqs
         self.device = device
+        self.bucket = bucket             # of the longest context this graph is replayed for (context.split_bucket)
         self.n_seqs = b
         self.n_tokens = b
         self.max_q_len = 1
@@ -75,7 +76,7 @@ class _StaticContext:
     def decode_workspace(self, n_heads: int, head_dim: int, n_kv_heads: int = 1):
         key = (n_heads, head_dim, n_kv_heads)
         if key not in self._workspaces:
-            n_splits = decode_splits(self.n_seqs, n_kv_heads)
+            n_splits = decode_splits(self.n_seqs, n_kv_heads, self.bucket)
             ws = torch.empty(self.n_seqs * n_heads * n_splits * (head_dim + 2), dtype=torch.float32,
                              device=self.device)
             self._workspaces[key] = (n_splits, ws)
@@ -86,13 +87,14 @@ class _StaticContext:
 
 
 class DecodeGraph:
-    """One captured decode step for a fixed number of sequences."""
+    """One captured decode step for a fixed number of sequences and a fixed split count of
+    decode attention (the grid of a captured launch cannot change)."""
 
-    def __init__(self, engine, n_seqs: int):
+    def __init__(self, engine, n_seqs: int, bucket: int = 16):
         self.engine = engine
         self.n_seqs = n_seqs
         width = max(1, pages_for(engine.max_seq_len))
-        self.ctx = _StaticContext(engine.device, n_seqs, [id(g) for g in engine.cache.kv_groups], width)
+        self.ctx = _StaticContext(engine.device, n_seqs, [id(g) for g in engine.cache.kv_groups], width, bucket)
         self.tokens_out = torch.zeros(n_seqs, dtype=torch.int32, device=engine.device)
         self.logits: Optional[torch.Tensor] = None
         self.graph: Optional[torch.cuda.CUDAGraph] = None

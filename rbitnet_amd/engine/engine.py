@@ -49,7 +49,7 @@ class Engine:
                            dtype=self.dtype, device=self.device, readers=model.cache_readers())
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0}
         self.use_graphs = bool(model.graph_safe)
-        self._graphs: Dict[int, Any] = {}
+        self._graphs: Dict[Tuple[int, int], Any] = {}      # (sequences, split bucket) -> DecodeGraph
         from ..sampling import Sampler
         self.sampler = Sampler(self.lib, self.device)
 
@@ -186,13 +186,15 @@ class Engine:
         if not self.use_graphs:
             logits = self.step([(s, [t]) for s, t in zip(slots, tokens)], "last")
             return self.sampler.sample(logits, temperatures, uniforms)
+        from .context import split_bucket
         from .decode_graph import DecodeGraph
         n = len(slots)
-        if n not in self._graphs:
+        key = (n, split_bucket(max(self.cache.length(s) for s in slots) + 1))
+        if key not in self._graphs:
             if len(self._graphs) >= 24:
                 self._graphs.pop(next(iter(self._graphs)))
-            self._graphs[n] = DecodeGraph(self, n)
-        out = self._graphs[n].run(slots, tokens, temperatures, uniforms)
+            self._graphs[key] = DecodeGraph(self, n, key[1])
+        out = self._graphs[key].run(slots, tokens, temperatures, uniforms)
         self.stats["steps"] += 1
         self.stats["decode_tokens"] += n
         return out

@@ -31,7 +31,7 @@ from .linear import linear
 
 DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight"}
 _MATRIX_CORE_HEAD_DIMS = (64, 128)
-_DECODE_GROUPS = (1, 2, 4, 8)           # query heads per kv head the decode kernels are built for
+_DECODE_GROUPS = tuple(range(1, 17))    # query heads per kv head the decode kernels take
 
 
 class Attention(Part):

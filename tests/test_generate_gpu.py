@@ -195,7 +195,7 @@ def test_graph_decode_equals_launch_by_launch(dtype):
             toks = eng.decode_step(slots, toks, temps, us)
             hist.append(list(toks))
             if eng.use_graphs:
-                g = eng._graphs[len(slots)]
+                g = next(gr for (n, _), gr in eng._graphs.items() if n == len(slots))
                 hist.append(g.logits.float().cpu().clone())
                 torch.cuda.synchronize()
                 _ = (torch.ones(1000, device="cuda") * 2).sum().item()      # unrelated eager work

@@ -276,9 +276,22 @@ def test_attention_prefill_bf16(lib, n_heads, n_kv, d, window):
     assert _rel(out, want) < 1.5e-2
 
 
-@pytest.mark.parametrize("n_heads,n_kv,d,window,n_splits", [(4, 1, 128, 0, 3), (8, 8, 64, 0, 1), (8, 4, 128, 0, 8),
-                                                           (8, 1, 64, 90, 2), (2, 2, 128, 65, 5)])
-def test_attention_decode_bf16(lib, n_heads, n_kv, d, window, n_splits):
+@pytest.fixture
+def decode_kernel(lib, request):
+    """"auto": the kernel the library picks for the group size; "matrix": the matrix-core
+    decode kernel whatever the group size."""
+    lib._lib.rb_tune_decode_mfma(1 if request.param == "matrix" else 0)
+    yield request.param
+    lib._lib.rb_tune_decode_mfma(0)
+
+
+_DECODE_CASES = [(4, 1, 128, 0, 3), (8, 8, 64, 0, 1), (8, 4, 128, 0, 8), (8, 1, 64, 90, 2), (2, 2, 128, 65, 5),
+                 (6, 2, 128, 0, 3), (16, 1, 64, 0, 2), (10, 2, 128, 70, 2), (7, 1, 64, 0, 4), (12, 1, 128, 130, 1)]
+
+
+@pytest.mark.parametrize("decode_kernel", ["auto", "matrix"], indirect=True)
+@pytest.mark.parametrize("n_heads,n_kv,d,window,n_splits", _DECODE_CASES)
+def test_attention_decode_bf16(lib, n_heads, n_kv, d, window, n_splits, decode_kernel):
     past, q_lens = [0, 70, 129, 63, 64, 300], [1, 1, 1, 1, 1, 1]
     dtype = torch.bfloat16
     g, bt, tok_seq, tok_pos, total = _paged_setup(past, q_lens, n_kv, d, dtype, seed=n_heads + 1)
@@ -316,9 +329,14 @@ def test_far_key_stands_out(lib):
                               bt.to(DEV), n_heads, n_kv, d, scale, 0)
         outs.append(out.clone())
         ws = torch.empty(n_heads * 4 * (d + 2), device=DEV)
-        lib.attention_decode_bf16(q.to(dtype).to(DEV), kp.to(DEV), vp.to(DEV), out, tok_pos.to(DEV), bt.to(DEV),
-                                  n_heads, n_kv, d, scale, 0, 4, ws)
-        outs.append(out.clone())
+        for mode in (0, 1):             # the vector kernel, the matrix-core kernel
+            lib._lib.rb_tune_decode_mfma(mode)
+            try:
+                lib.attention_decode_bf16(q.to(dtype).to(DEV), kp.to(DEV), vp.to(DEV), out, tok_pos.to(DEV),
+                                          bt.to(DEV), n_heads, n_kv, d, scale, 0, 4, ws)
+            finally:
+                lib._lib.rb_tune_decode_mfma(0)
+            outs.append(out.clone())
         cu = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
         lib.attention_prefill_bf16(q.to(dtype).to(DEV), kp.to(DEV), vp.to(DEV), out, cu,
                                    torch.tensor([total - 1], dtype=torch.int32, device=DEV), bt.to(DEV), 1, 1,
@@ -350,10 +368,10 @@ def test_sample_greedy_and_inverse_cdf(lib):
         assert tokens[r].item() == sample_token(row, float(temps[r]), float(us[r])), r
 
 
+@pytest.mark.parametrize("decode_kernel", ["auto", "matrix"], indirect=True)
 @pytest.mark.parametrize("style", [0, 1])
-@pytest.mark.parametrize("n_heads,n_kv,d,window,n_splits", [(4, 1, 128, 0, 3), (8, 8, 64, 0, 1), (8, 4, 128, 0, 8),
-                                                           (8, 1, 64, 90, 2), (2, 2, 128, 65, 5), (4, 2, 64, 0, 32)])
-def test_attention_decode_fused_bf16(lib, n_heads, n_kv, d, window, n_splits, style):
+@pytest.mark.parametrize("n_heads,n_kv,d,window,n_splits", _DECODE_CASES + [(4, 2, 64, 0, 32)])
+def test_attention_decode_fused_bf16(lib, n_heads, n_kv, d, window, n_splits, style, decode_kernel):
     """Rotation, cache write and attention in one kernel (and the combination of splits),
     against the separate steps computed plainly; called three times in a row."""
     past, q_lens = [0, 70, 129, 63, 64, 300], [1, 1, 1, 1, 1, 1]
@@ -441,12 +459,16 @@ def test_attention_long_context(lib):
     kp, vp = kp.to(DEV), vp.to(DEV)
     scale = 1 / math.sqrt(d)
     want = _attention_ref(q, k_full, v_full, tok_seq, tok_pos, n_heads, n_kv, scale, 0)
-    for n_splits in (1, 3, 16):
+    for n_splits, mode in ((1, 0), (3, 0), (16, 0), (1, 1), (5, 1), (16, 1)):
         out = torch.full((2, n_heads * d), float("nan"), dtype=dtype, device=DEV)
         ws = torch.empty(2 * n_heads * n_splits * (d + 2), device=DEV)
-        lib.attention_decode_bf16(q.to(DEV), kp, vp, out, tok_pos.to(DEV), bt.to(DEV), n_heads, n_kv, d, scale, 0,
-                                  n_splits, ws)
-        assert _rel(out, want) < 1e-2, n_splits
+        lib._lib.rb_tune_decode_mfma(mode)             # 1: the matrix-core kernel
+        try:
+            lib.attention_decode_bf16(q.to(DEV), kp, vp, out, tok_pos.to(DEV), bt.to(DEV), n_heads, n_kv, d, scale,
+                                      0, n_splits, ws)
+        finally:
+            lib._lib.rb_tune_decode_mfma(0)
+        assert _rel(out, want) < 1e-2, (n_splits, mode)
     # a 100-token step on top of 4000 cached tokens
     past, q_lens = [4000], [100]
     g, bt, tok_seq, tok_pos, total = _paged_setup(past, q_lens, n_kv, d, dtype, n_pages=160, seed=10)
