@@ -585,8 +585,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 // (keys 4 grp + 0..3 of two tiles) are its operand, and V^T is read in the same order.
 // Rows of the last page beyond the position may hold anything (0 x NaN would spoil the
 // product): they are cleared in LDS, and the token's own row is put there (FUSED).
-template <int D, bool FUSED>
-__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
+template <int D, int NW, bool FUSED>
+__global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
     const float* __restrict__ qkv, const bf16_t* __restrict__ q_in, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int style, bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
@@ -599,13 +599,14 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   constexpr int VI = RB_PAGE / RPI;   // direct load instructions per page
   constexpr int DL = D / 64;          // elements of a row per lane
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  uint16_t* vpages = reinterpret_cast<uint16_t*>(smem);                    // [4 waves][64 keys][D]
-  uint16_t* q_h = vpages + 4 * RB_PAGE * D;                                // [16][D]
+  constexpr int NT = 64 * NW;
+  uint16_t* vpages = reinterpret_cast<uint16_t*>(smem);                    // [NW waves][64 keys][D]
+  uint16_t* q_h = vpages + NW * RB_PAGE * D;                               // [16][D]
   uint16_t* knew_h = q_h + 16 * D;
   uint16_t* vnew_h = knew_h + D;
-  float* red_m = reinterpret_cast<float*>(vnew_h + D);                     // [4][16]
-  float* red_l = red_m + 64;                                               // [4][64]
-  float* red_acc = reinterpret_cast<float*>(smem);                         // [4][16][D], over the pages at the end
+  float* red_m = reinterpret_cast<float*>(vnew_h + D);                     // [NW][16]
+  float* red_l = red_m + NW * 16;                                          // [NW][64]
+  float* red_acc = reinterpret_cast<float*>(smem);                         // [NW][16][D], over the pages at the end
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // the same for the whole wave: LDS addresses go to a scalar register
@@ -623,7 +624,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const float* src = qkv + (size_t)b * row_width;
     const float* cr = cos_t ? cos_t + (size_t)pos * HALF : nullptr;
     const float* sr = cos_t ? sin_t + (size_t)pos * HALF : nullptr;
-    for (int idx = tid; idx < 17 * HALF; idx += 256) {
+    for (int idx = tid; idx < 17 * HALF; idx += NT) {
       const int gg = idx / HALF, i = idx - gg * HALF;
       const int i0 = style == 0 ? 2 * i : i, i1 = style == 0 ? 2 * i + 1 : i + HALF;
       uint16_t* dst = gg < 16 ? q_h + gg * D : knew_h;
@@ -643,9 +644,9 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
       dst[i0] = f32_to_bf16_bits(y0);
       dst[i1] = f32_to_bf16_bits(y1);
     }
-    for (int d = tid; d < D; d += 256) vnew_h[d] = f32_to_bf16_bits(src[(size_t)(n_heads + n_kv + kvh) * D + d]);
+    for (int d = tid; d < D; d += NT) vnew_h[d] = f32_to_bf16_bits(src[(size_t)(n_heads + n_kv + kvh) * D + d]);
   } else {
-    for (int idx = tid; idx < 16 * D; idx += 256) {
+    for (int idx = tid; idx < 16 * D; idx += NT) {
       const int gg = idx / D, d = idx - gg * D;
       q_h[idx] = gg < G ? q_in[((size_t)b * n_heads + kvh * G + gg) * D + d].bits : (uint16_t)0;
     }
@@ -654,7 +655,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   if (FUSED && split == (last_page - first_page) % n_splits) {      // this workgroup owns the last page
     const int page = pages[last_page];
     const size_t at = ((size_t)page * n_kv + kvh) * RB_PAGE * D + (size_t)(pos % RB_PAGE) * D;
-    for (int d = tid; d < D; d += 256) {
+    for (int d = tid; d < D; d += NT) {
       k_pages[at + d].bits = knew_h[d];
       v_pages[at + d].bits = vnew_h[d];
     }
@@ -670,7 +671,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   uint16_t* vpage = vpages + wave * RB_PAGE * D;
   const uint32_t vpage_lds = (uint32_t)(uintptr_t)vpage;
 
-  for (int pg = first_page + split + n_splits * wave; pg <= last_page; pg += 4 * n_splits) {
+  for (int pg = first_page + split + n_splits * wave; pg <= last_page; pg += NW * n_splits) {
     const int page = __builtin_amdgcn_readfirstlane(pages[pg]);
     const size_t base = ((size_t)page * n_kv + kvh) * RB_PAGE * D;
     // the reads of the previous page have all returned before its area is overwritten
@@ -776,7 +777,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     }
   }
 
-  // ---- the four waves' states into one (the pages' area is reused for the outputs)
+  // ---- the waves' states into one (the pages' area is reused for the outputs)
   __syncthreads();
   if (c16 < G) {
 #pragma unroll
@@ -787,15 +788,15 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   red_l[wave * 64 + lane] = l_part;
   if (grp == 0) red_m[wave * 16 + c16] = m_run;
   __syncthreads();
-  for (int idx = tid; idx < G * D; idx += 256) {
+  for (int idx = tid; idx < G * D; idx += NT) {
     const int gg = idx / D, d = idx % D;
     float mx = red_m[gg];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) mx = fmaxf(mx, red_m[w * 16 + gg]);
+    for (int w = 1; w < NW; ++w) mx = fmaxf(mx, red_m[w * 16 + gg]);
     const float m_safe = (mx == -INFINITY) ? 0.f : mx;
     float a = 0.f, l = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NW; ++w) {
       const float f = exp2f(red_m[w * 16 + gg] - m_safe);
       a += red_acc[((size_t)w * 16 + gg) * D + d] * f;
       const float* lw = red_l + w * 64 + gg;
@@ -857,10 +858,10 @@ static void launch_decode(const DecodeArgs& a, hipStream_t s) {
   if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits);
 }
 
-template <int D, bool FUSED>
-static int launch_decode_mfma(const DecodeArgs& a, hipStream_t s) {
-  const size_t lds = (size_t)4 * RB_PAGE * D * 2 + 16 * D * 2 + 2 * D * 2 + (64 + 256) * sizeof(float);
-  auto kern = attn_decode_mfma_kernel<D, FUSED>;
+template <int D, int NW, bool FUSED>
+static int launch_decode_mfma_nw(const DecodeArgs& a, hipStream_t s) {
+  const size_t lds = (size_t)NW * RB_PAGE * D * 2 + 16 * D * 2 + 2 * D * 2 + (size_t)NW * (16 + 64) * sizeof(float);
+  auto kern = attn_decode_mfma_kernel<D, NW, FUSED>;
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -869,10 +870,22 @@ static int launch_decode_mfma(const DecodeArgs& a, hipStream_t s) {
     configured = true;
   }
   dim3 grid(a.n_splits, a.n_kv, a.n_seqs);
-  kern<<<grid, 256, lds, s>>>(a.qkv, a.q, a.cos_t, a.sin_t, a.style, a.k, a.v, a.out, a.tok_pos, a.bt, a.bt_stride,
-                              a.n_heads, a.n_kv, a.sl2, a.window, a.n_splits, a.ws);
+  kern<<<grid, 64 * NW, lds, s>>>(a.qkv, a.q, a.cos_t, a.sin_t, a.style, a.k, a.v, a.out, a.tok_pos, a.bt,
+                                  a.bt_stride, a.n_heads, a.n_kv, a.sl2, a.window, a.n_splits, a.ws);
   if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits);
   return 0;
+}
+
+// 8 waves (8 pages at a time) while that still gives every workgroup a compute unit of its
+// own (a wave's page of V takes 16 KB of LDS at head size 128), else 4 waves and two
+// workgroups per compute unit.
+static int g_decode_waves = 0;
+extern "C" void rb_tune_decode_waves(int nw) { g_decode_waves = nw; }      // experiments only; 0 = built-in
+template <int D, bool FUSED>
+static int launch_decode_mfma(const DecodeArgs& a, hipStream_t s) {
+  const long long wgs = (long long)a.n_splits * a.n_kv * a.n_seqs;
+  const int nw = g_decode_waves ? g_decode_waves : (wgs <= 256 ? 8 : 4);
+  return nw == 8 ? launch_decode_mfma_nw<D, 8, FUSED>(a, s) : launch_decode_mfma_nw<D, 4, FUSED>(a, s);
 }
 
 // Which decode kernel: 0 = by group size (matrix cores from 2 query heads per kv head on: the

@@ -71,8 +71,11 @@ class Model:
         self.device = torch.device(device)
         self.lib = lib
 
+        shared: Dict = {}
+
         def env_for(i: int) -> BuildEnv:
-            env = BuildEnv(hidden_size=spec.hidden_size, dtype=dtype, device=self.device, lib=lib, layer_index=i)
+            env = BuildEnv(hidden_size=spec.hidden_size, dtype=dtype, device=self.device, lib=lib, layer_index=i,
+                           shared=shared)
             env.generic_only = generic_only
             return env
 

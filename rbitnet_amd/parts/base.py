@@ -46,6 +46,9 @@ class BuildEnv:
     device: torch.device
     lib: Any                    # rbitnet_amd.csrc.lib.Kernels (None when only shapes are wanted)
     layer_index: int = -1
+    # one dictionary for all layers of a model: read-only data (tables) that parts with equal
+    # parameters build once and share, keyed by the part
+    shared: Dict[Any, Any] = field(default_factory=dict)
 
 
 @dataclass

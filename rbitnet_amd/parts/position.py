@@ -66,9 +66,15 @@ class Rope(Part):
         self.cos: Optional[torch.Tensor] = None
         self.sin: Optional[torch.Tensor] = None
         if env.lib is not None:
-            angles = torch.arange(self.max_positions, dtype=torch.float64)[:, None] * inv[None, :]
-            self.cos = torch.cos(angles).to(torch.float32).to(env.device).contiguous()
-            self.sin = torch.sin(angles).to(torch.float32).to(env.device).contiguous()
+            # one table for all layers with the same rotation: a step's row is then fetched
+            # from memory once and found in cache by the layers after the first
+            key = ("rope", self.head_dim, float(params["theta"]), repr(sorted((params.get("scaling") or {}).items())),
+                   self.max_positions, str(env.device))
+            if key not in env.shared:
+                angles = torch.arange(self.max_positions, dtype=torch.float64)[:, None] * inv[None, :]
+                env.shared[key] = (torch.cos(angles).to(torch.float32).to(env.device).contiguous(),
+                                   torch.sin(angles).to(torch.float32).to(env.device).contiguous())
+            self.cos, self.sin = env.shared[key]
 
     def rotation_tables(self):
         """(cos, sin, pairing style): lets a mixer fold the rotation into its own kernel."""
