@@ -50,6 +50,8 @@ class Engine:
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0}
         self.use_graphs = bool(model.graph_safe)
         self._graphs: Dict[Tuple[int, int], Any] = {}      # (sequences, split bucket) -> DecodeGraph
+        # float32 [sequences, vocab] of the last `decode_step`, valid until the next one
+        self.last_decode_logits: Optional[torch.Tensor] = None
         from ..sampling import Sampler
         self.sampler = Sampler(self.lib, self.device)
 
@@ -185,6 +187,7 @@ class Engine:
                 raise InferenceError(f"slot {s}: sequence position >= max_seq ({self.max_seq_len})")
         if not self.use_graphs:
             logits = self.step([(s, [t]) for s, t in zip(slots, tokens)], "last")
+            self.last_decode_logits = logits
             return self.sampler.sample(logits, temperatures, uniforms)
         from .context import split_bucket
         from .decode_graph import DecodeGraph
@@ -195,6 +198,7 @@ class Engine:
                 self._graphs.pop(next(iter(self._graphs)))
             self._graphs[key] = DecodeGraph(self, n, key[1])
         out = self._graphs[key].run(slots, tokens, temperatures, uniforms)
+        self.last_decode_logits = self._graphs[key].logits
         self.stats["steps"] += 1
         self.stats["decode_tokens"] += n
         return out

@@ -32,7 +32,14 @@ TINY_C = {
     "vocab_size": 500, "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 512,
     "tie_word_embeddings": False, "rope_style": "half",
 }
-CONFIGS = {"A": (TINY_A, 0, 0.02), "B": (TINY_B, 1, 0.0), "C": (TINY_C, 2, 0.02)}
+# one layer with room for a thousand positions, for what only long contexts show
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 128, "num_hidden_layers": 1,
+    "num_attention_heads": 4, "num_key_value_heads": 1, "head_dim": 64, "intermediate_size": 208,
+    "vocab_size": 300, "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 1088,
+    "tie_word_embeddings": True,
+}
+CONFIGS = {"A": (TINY_A, 0, 0.02), "B": (TINY_B, 1, 0.0), "C": (TINY_C, 2, 0.02), "D": (TINY_D, 3, 0.02)}
 
 _FOLDERS = {}
 _TMP = None

@@ -95,6 +95,33 @@ def test_long_decoding(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_where_the_split_count_changes(dtype):
+    """Decode attention deals a sequence's pages to more workgroups as the context grows (one
+    split up to 15 pages, two from 16 pages on), and the captured step is kept per split
+    count.  Logits from 940 to 990 keys against the plain implementation, replayed as
+    graphs and launched one by one."""
+    name = "D"
+    toks = tokens_for(name, 990, 5)
+    want = plain_logits(name, tuple(toks))
+    for graphs in (True, False):
+        eng = _engine(name, dtype, max_tokens=1088, max_batch=1)
+        assert eng.use_graphs
+        eng.use_graphs = graphs
+        slot = eng.alloc_slot()
+        assert eng.step([(slot, toks[:940])], [[]]).shape[0] == 0
+        rows = []
+        for t in toks[940:]:
+            eng.decode_step([slot], [t])
+            rows.append(eng.last_decode_logits.float().cpu().clone())
+        if graphs:
+            assert sorted(b for _, b in eng._graphs) == [1, 2]
+        eng.free_slot(slot)
+        got = torch.cat(rows).double()
+        err = (got - want[940:]).abs().amax(dim=1) / want.abs().max()
+        assert float(err.max()) < TOL[dtype], f"graphs={graphs}: worst position {940 + int(err.argmax())}: {float(err.max())}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_first_tokens_of_a_sequence(name, dtype):
     """Positions 0, 1, 2 alone and together: a one-token sequence attends to itself only."""
