@@ -585,6 +585,27 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 // (keys 4 grp + 0..3 of two tiles) are its operand, and V^T is read in the same order.
 // Rows of the last page beyond the position may hold anything (0 x NaN would spoil the
 // product): they are cleared in LDS, and the token's own row is put there (FUSED).
+// ds_read_b64_tr_b16: every lane gives the address of 4 consecutive 16-bit values; within each
+// group of 16 lanes, lane j receives value j % 4 of lanes j / 4, j / 4 + 4, j / 4 + 8, j / 4 + 12.
+typedef __attribute__((ext_vector_type(4))) short i16x4_t;
+__device__ __forceinline__ uint2 lds_read_transposed(const uint16_t* p) {
+  union {
+    i16x4_t v;
+    uint2 u;
+  } r;
+  r.v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(p));
+  return r.u;
+}
+// Which 16-byte chunk of a row of V a chunk is stored in is chunk ^ v_swizzle(key): a
+// transposing read touches 16 consecutive keys at the same 32 bytes of their rows, and the
+// swizzle spreads them over the 8 bank windows of 32 bytes (twice each: the read takes two
+// cycles anyway).  Rows of 256 bytes (D = 128) all start at bank 0; of rows of 128 bytes
+// (D = 64) every second one does.
+template <int D>
+__device__ __forceinline__ int v_swizzle(int key) {
+  return D == 128 ? ((key & 7) << 1) : (((key >> 1) & 3) << 1);
+}
+
 template <int D, int NW, bool FUSED>
 __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
     const float* __restrict__ qkv, const bf16_t* __restrict__ q_in, const float* __restrict__ cos_t,
@@ -679,7 +700,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < VI; ++i) {
       const int key = i * RPI + lane / CPR;
-      const int chunk = (lane % CPR) ^ ((key >> 2) & 3);
+      const int chunk = (lane % CPR) ^ v_swizzle<D>(key);
       load_to_lds16(v_pages + base, (uint32_t)(key * D + chunk * 8) * 2u, vpage_lds + i * 1024u);
     }
     Frag8 kf[4][KS];
@@ -748,7 +769,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
       const int r_pos = pos % RB_PAGE;
       for (int row = FUSED ? r_pos : r_pos + 1; row < RB_PAGE; ++row) {
         const int d = lane * DL;
-        uint16_t* dst = vpage + row * D + (((d >> 3) ^ ((row >> 2) & 3)) * 8 + (d & 7));
+        uint16_t* dst = vpage + row * D + (((d >> 3) ^ v_swizzle<D>(row)) * 8 + (d & 7));
         const bool own = FUSED && row == r_pos;
         if (DL == 2)
           *reinterpret_cast<uint32_t*>(dst) = own ? *reinterpret_cast<const uint32_t*>(vnew_h + d) : 0u;
@@ -756,22 +777,30 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
           *dst = own ? vnew_h[d] : (uint16_t)0;
       }
     }
-    // ---- O^T[d, head] += V^T P^T: lane reads, for d = 16 dt + c16, the 8 keys of its group
+    // ---- O^T[d, head] += V^T P^T.  A transposing LDS read hands every lane of a 16-lane group 4
+    // keys of its own d: lane i of the group points at 4 consecutive d (4 (i % 4) ..) of key
+    // i / 4, and lane j receives element j % 4 of lanes j / 4, j / 4 + 4, ...: keys 0..3 at d = j.
+    // Two of them make the 8 keys of the group's MFMA operand.
+    const int key_in = c16 >> 2;                       // which of the 4 keys this lane points at
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      const int d = 16 * dt + c16;
-      const uint16_t* col = vpage + (size_t)(4 * grp) * D + (((d >> 3) ^ grp) * 8 + (d & 7));
+      const int d4 = 16 * dt + 4 * (c16 & 3);
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        uint32_t wv[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          // pairs (e = 0, 1 of tile 2 s2; e = 2, 3: of tile 2 s2 + 1): keys 32 s2 + 16 (e / 2) + 4 grp + 2 (e % 2) + 0, 1
-          const int key0 = 32 * s2 + 16 * (e / 2) + 2 * (e % 2);
-          wv[e] = (uint32_t)col[(size_t)key0 * D] | ((uint32_t)col[(size_t)(key0 + 1) * D] << 16);
-        }
         Frag8 vf;
-        vf.u = make_uint4(wv[0], wv[1], wv[2], wv[3]);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int key = 32 * s2 + 16 * h + 4 * grp + key_in;
+          const uint16_t* src = vpage + key * D + (((d4 >> 3) ^ v_swizzle<D>(key)) * 8 + (d4 & 7));
+          const uint2 got = lds_read_transposed(src);
+          if (h == 0) {
+            vf.u.x = got.x;
+            vf.u.y = got.y;
+          } else {
+            vf.u.z = got.x;
+            vf.u.w = got.y;
+          }
+        }
         acc_o[dt] = mfma16(vf, pf[s2], acc_o[dt]);
       }
     }
