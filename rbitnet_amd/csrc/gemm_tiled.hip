@@ -250,6 +250,7 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   constexpr int LOADS = W_LOADS + X_LOADS;      // per thread and stage
   constexpr int STAGE = (BN + BM) * BK;         // elements
   static_assert(BN % (RPW * NWAVES) == 0 && BM % (RPW * NWAVES) == 0, "tile does not divide among the waves");
+  static_assert(WN % 32 == 0 && WM % 32 == 0 && BN % WN == 0 && BM % WM == 0, "wave tiles are made of 32 x 32 pieces");
   static_assert(S >= 2 && LOADS * (S - 1) < 64, "too many loads in flight for the counter");
   bf16_t* lds = reinterpret_cast<bf16_t*>(smem);
 
@@ -470,8 +471,8 @@ static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, in
 // Which tile for which product.  Measured on the Llama-3-8B products at M = 2048 .. 8192: the
 // kernels are bound by what they pull from L2 and LDS (a 128 x 128 x 64 tile needs a byte per
 // 64 flop, a 256 x 256 one half of that), so the largest tile that still gives every compute
-// unit work wins: 256 x 256 when there are at least ~160 such tiles, else 128 x 128 (two
-// workgroups per compute unit).  The direct-to-LDS kernel is 10-20 % faster than the one that
+// unit work wins: 256 x 256 (or 192 x 256) when there are at least ~160 such tiles, else
+// 128 x 128 (two workgroups per compute unit).  The direct-to-LDS kernel is 10-20 % faster than the one that
 // stages tiles in registers and is used whenever K is a multiple of its 64-deep tile.
 template <int EPI, typename TO>
 static int launch_tiled(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
@@ -480,12 +481,22 @@ static int launch_tiled(const bf16_t* x, const bf16_t* w, void* c, int m, int n,
     const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
     const long long t256x128 = (long long)((m + 127) / 128) * ((n + 255) / 256);
     const bool dma = k % 64 == 0 && (long long)k * 512 < (1LL << 32);
-    if (dma) cfg = t256 >= 160 ? 4 : 5;
+    if (dma && t256 >= 160) {
+      // 256 x 256 tiles, or 192 rows of W by 256 tokens when that fills the last round of
+      // workgroups better: rounds of 256 workgroups times the time of a tile (a 192-row tile
+      // does 0.75 of the work in 0.81 of the time)
+      const long long t192 = (long long)((m + 255) / 256) * ((n + 191) / 192);
+      const long long cost256 = (t256 + 255) / 256 * 1000, cost192 = (t192 + 255) / 256 * 815;
+      cfg = cost192 < cost256 ? 6 : 4;
+    } else if (dma) {
+      cfg = 5;
+    }
     else if (t256 >= 160) cfg = 3;
     else if (k >= 8192 && t256x128 >= 200) cfg = 2;
     else cfg = 1;
   }
   switch (cfg) {
+    case 6: return launch_dma_cfg<192, 256, 96, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
     case 5: return launch_dma_cfg<128, 128, 64, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
     case 4: return launch_dma_cfg<256, 256, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
     case 3: return launch_tiled_cfg<256, 256, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);

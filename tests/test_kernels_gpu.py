@@ -87,11 +87,13 @@ def test_gemm_bf16_gated(lib, m, ff, k):
 
 
 @pytest.mark.parametrize("m,n,k,gated", [(513, 300, 128, False), (700, 14000, 192, False), (700, 14000, 64, False),
-                                         (257, 41000, 320, False), (600, 14016, 128, True), (130, 96, 64, True)])
+                                         (257, 41000, 320, False), (600, 14016, 128, True), (130, 96, 64, True),
+                                         (1024, 16384, 128, False), (1000, 16384, 64, True)])
 def test_gemm_bf16_tiles_loaded_straight_into_lds(lib, m, n, k, gated):
     """K a multiple of 64 and more than 64 tokens: the kernels whose tiles go from memory into
-    LDS without passing registers, with both tile sizes, partial tiles at both edges, and as
-    few K tiles as one (fewer than the stages of the pipeline)."""
+    LDS without passing registers, with all three tile sizes (128 x 128; 256 x 256 when its
+    tiles fill whole rounds of workgroups, as with 4 x 64 of them; else 192 x 256), partial
+    tiles at both edges, and as few K tiles as one (fewer than the stages of the pipeline)."""
     from rbitnet_amd.parts.linear import pack_gate_up
     g = torch.Generator().manual_seed(m + n + k)
     x = torch.randn(m, k, generator=g).bfloat16()
