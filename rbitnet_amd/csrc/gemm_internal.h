@@ -12,11 +12,9 @@ int gemm_skinny_launch(const bf16_t* x, const bf16_t* w, void* c, int dtype_out,
 // sizes are not for it and nothing was launched
 bool gemm_resident_try(const bf16_t* x, const bf16_t* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
                        hipStream_t s, int* rc);
-// more than 64 tokens: tiles through LDS (gemm_tiled.hip)
-int gemm_tiled_launch(const bf16_t* x, const bf16_t* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
-                      hipStream_t s);
-// 17..64 tokens with K % 64 == 0: one token tile, K cut into gemm_stream_parts(...) slices
-// (0: not for this kernel; more than 1: needs parts * m * n floats of workspace)
-int gemm_stream_parts(int m, int n, int k, int epilogue);
-int gemm_stream_launch(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int dtype_out, int epilogue,
-                       int m, int n, int k, hipStream_t s);
+// more than 16 tokens (more than 64 when K is no multiple of 64): tiles through LDS
+// (gemm_tiled.hip).  gemm_tiled_parts: 0 when these sizes are not for it, else the number of K
+// slices it will use; more than 1 needs parts * m * n floats of workspace.
+int gemm_tiled_parts(int m, int n, int k, int epilogue);
+int gemm_tiled_launch(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int dtype_out, int epilogue, int m,
+                      int n, int k, hipStream_t s);

@@ -2,18 +2,23 @@
 // accumulation: picks the kernel for the sizes.
 //  * at most 16 tokens: W streamed straight into MFMA operands (gemm_skinny.hip); with more
 //    than 8192 rows of W the variant that keeps the tokens in registers.
-//  * 17..64 tokens: one token tile, W streamed through LDS (gemm_tiled.hip); when K is no
-//    multiple of 64, the skinny kernel.
-//  * more: tiles through LDS (gemm_tiled.hip).
+//  * more: tiles of W and of the tokens through LDS, with K cut into slices over workgroups
+//    where the tiles alone are too few to fill the GPU (gemm_tiled.hip); 17..64 tokens with a
+//    K that is no multiple of 64: the skinny kernel.
 #include "api.h"
 #include "gemm_internal.h"
 
-static int g_use_resident = 1, g_use_stream = 1;
+static int g_use_resident = 1, g_use_tiled_small = 1;
 extern "C" void rb_tune_use_resident(int on) { g_use_resident = on; }      // experiments only
-extern "C" void rb_tune_use_stream(int on) { g_use_stream = on; }          // experiments only
+extern "C" void rb_tune_use_stream(int on) { g_use_tiled_small = on; }     // experiments only: 0 = skinny up to 64 tokens
+
+static int tiled_parts(int m, int n, int k, int epilogue) {
+  if (m <= 64 && !g_use_tiled_small) return 0;
+  return gemm_tiled_parts(m, n, k, epilogue);
+}
 
 extern "C" long long rb_gemm_workspace_floats(int m, int n, int k, int epilogue) {
-  const int p = g_use_stream ? gemm_stream_parts(m, n, k, epilogue) : 0;
+  const int p = tiled_parts(m, n, k, epilogue);
   return p > 1 ? (long long)p * m * n : 0;
 }
 
@@ -29,10 +34,8 @@ extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out
   const bf16_t* xa = (const bf16_t*)a;
   const bf16_t* wa = (const bf16_t*)w;
   int rc = 0;
-  if (m > 64) {
-    rc = gemm_tiled_launch(xa, wa, c, dtype_out, epilogue, m, n, k, s);
-  } else if (g_use_stream && gemm_stream_parts(m, n, k, epilogue) >= 1) {
-    rc = gemm_stream_launch(xa, wa, c, workspace, dtype_out, epilogue, m, n, k, s);
+  if (tiled_parts(m, n, k, epilogue) >= 1) {
+    rc = gemm_tiled_launch(xa, wa, c, workspace, dtype_out, epilogue, m, n, k, s);
   } else if (!(g_use_resident && m <= 16 && n > 8192 &&
                gemm_resident_try(xa, wa, c, dtype_out, epilogue, m, n, k, s, &rc))) {
     rc = gemm_skinny_launch(xa, wa, c, dtype_out, epilogue, m, n, k, s);

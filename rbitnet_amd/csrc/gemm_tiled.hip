@@ -407,45 +407,6 @@ static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int 
   return 0;
 }
 
-// ------------------------------------------------------------------ 17 .. 64 tokens, K % 64 == 0
-// The same kernel with one token tile: W streams through LDS three stages deep, two
-// workgroups per compute unit.  Few rows of W: K is also cut into slices over workgroups
-// (grid.y); each slice writes its partial sums to its own [M, N] slab of a workspace, and
-// gemm_sum_slabs_kernel adds them up in a fixed order.
-static int g_stream_parts = 0;
-extern "C" void rb_tune_stream_parts(int parts) { g_stream_parts = parts; }      // experiments only; 0 = built-in
-
-static int stream_parts(int m, int n, int k, int epilogue) {
-  if (m <= 16 || m > 64 || k % 64 != 0 || (long long)k * 256 >= (1LL << 32)) return 0;      // not for this kernel
-  if (epilogue == 1) return 1;
-  const int tiles = (n + 127) / 128;
-  const int kt = k / 64;
-  if (g_stream_parts && kt % g_stream_parts == 0) return g_stream_parts;
-  // every slice writes and re-reads an [M, N] slab (8 bytes per element): keep that under half
-  // of W's bytes, the slices at 16 and at least 4 tiles deep, the workgroups at one per compute
-  // unit (more slices cost more in slabs than they gain: measured on N = 4096 and 6144)
-  int cap = k / (8 * m);
-  if (cap > 16) cap = 16;
-  int best = 1;
-  for (int p = 1; p <= cap; ++p) {
-    if (kt % p != 0 || kt / p < 4) continue;
-    if ((long long)tiles * p <= 256) best = p;
-  }
-  return best;
-}
-
-template <int EPI, typename TO>
-static int launch_stream(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int m, int n, int k,
-                         hipStream_t s) {
-  const int parts = stream_parts(m, n, k, EPI);
-  RB_REQUIRE(parts >= 1, "rb_gemm_bf16: internal: not a product for the streaming kernel");
-  RB_REQUIRE(parts == 1 || workspace != nullptr, "rb_gemm_bf16: M=%d N=%d K=%d needs a workspace of %lld floats", m, n,
-             k, (long long)parts * m * n);
-  return launch_dma_cfg<128, 64, 32, 64, 64, 3, EPI, TO>(x, w, c, m, n, k, s, parts, workspace);
-}
-
-static int g_tile_cfg = 0;
-extern "C" void rb_tune_tiles(int cfg) { g_tile_cfg = cfg; }      // experiments only; 0 = built-in choice
 
 template <int BN, int BM, int WN, int WM, int P, int EPI, typename TO>
 static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
@@ -468,56 +429,99 @@ static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, in
   return 0;
 }
 
-// Which tile for which product.  Measured on the Llama-3-8B products at M = 2048 .. 8192: the
-// kernels are bound by what they pull from L2 and LDS (a 128 x 128 x 64 tile needs a byte per
-// 64 flop, a 256 x 256 one half of that), so the largest tile that still gives every compute
-// unit work wins: 256 x 256 (or 192 x 256) when there are at least ~160 such tiles, else
-// 128 x 128 (two workgroups per compute unit).  The direct-to-LDS kernel is 10-20 % faster than the one that
-// stages tiles in registers and is used whenever K is a multiple of its 64-deep tile.
-template <int EPI, typename TO>
-static int launch_tiled(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
-  int cfg = g_tile_cfg;
-  if (cfg == 0) {
-    const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
+// ------------------------------------------------------------------ which tiles, how many K slices
+// Measured on the Llama-3-8B products (N = 4096 .. 28672, K = 4096 and 14336) from 17 to 8,192
+// tokens.  The kernels are bound by what they pull from L2 and LDS (a 128 x 128 x 64 tile needs
+// a byte per 64 flop, a 256 x 256 one half of that), so the largest tile that still gives
+// every compute unit work wins, and where even the smallest tiles are too few, K is cut into
+// slices over workgroups (grid.y): each slice writes its partial sums to its own [M, N] slab
+// of a workspace, and gemm_sum_slabs_kernel adds them up in a fixed order.
+//   cfg 4: 256 x 256 (8 waves)        at least ~160 such tiles
+//   cfg 6: 192 x 256 (8 waves)        ... when that fills the last round of workgroups better
+//   cfg 5: 128 x 128 (4 waves, 2 workgroups per compute unit)
+//   cfg 7: 128 rows of W x 64 tokens, 3 stages deep    up to 512 tokens, when cfg 5 has < 256 tiles
+//   cfg 1..3: tiles staged through registers, for K that is no multiple of 64 (more than 64 tokens)
+// Without K slices a product of 128 tokens by 4096 rows ran on 32 of the 256 compute units and
+// took as long as one of 768 tokens (K = 14336: 194 us; 41 us with 4 slices of 64-token tiles).
+struct TilePlan {
+  int cfg;        // 0: not for the kernels of this file
+  int parts;      // K slices; more than 1 needs parts * M * N floats of workspace
+};
+
+static int g_tile_cfg = 0, g_tile_parts = 0;
+extern "C" void rb_tune_tiles(int cfg, int parts) {       // experiments only; 0 = built-in choice
+  g_tile_cfg = cfg;
+  g_tile_parts = parts;
+}
+
+// The most slices that keep the workgroups within `slots`, the slices at least 4 tiles deep
+// and equal, and their number within `cap` (every slice writes and re-reads an [M, N] slab,
+// 8 bytes per element, against W's 2 N K bytes).
+static int k_slices(long long tiles, int k, int slots, int cap) {
+  const int kt = k / 64;
+  if (cap > 16) cap = 16;
+  int best = 1;
+  for (int p = 1; p <= cap; ++p)
+    if (kt % p == 0 && kt / p >= 4 && tiles * p <= slots) best = p;
+  return best;
+}
+
+static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
+  const bool dma = k % 64 == 0 && (long long)k * 512 < (1LL << 32);
+  const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
+  if (!dma) {
+    if (m <= 64) return {0, 1};
     const long long t256x128 = (long long)((m + 127) / 128) * ((n + 255) / 256);
-    const bool dma = k % 64 == 0 && (long long)k * 512 < (1LL << 32);
-    if (dma && t256 >= 160) {
-      // 256 x 256 tiles, or 192 rows of W by 256 tokens when that fills the last round of
-      // workgroups better: rounds of 256 workgroups times the time of a tile (a 192-row tile
-      // does 0.75 of the work in 0.81 of the time)
-      const long long t192 = (long long)((m + 255) / 256) * ((n + 191) / 192);
-      const long long cost256 = (t256 + 255) / 256 * 1000, cost192 = (t192 + 255) / 256 * 815;
-      cfg = cost192 < cost256 ? 6 : 4;
-    } else if (dma) {
-      cfg = 5;
-    }
-    else if (t256 >= 160) cfg = 3;
-    else if (k >= 8192 && t256x128 >= 200) cfg = 2;
-    else cfg = 1;
+    if (g_tile_cfg >= 1 && g_tile_cfg <= 3) return {g_tile_cfg, 1};
+    return {t256 >= 160 ? 3 : (k >= 8192 && t256x128 >= 200 ? 2 : 1), 1};
   }
-  switch (cfg) {
-    case 6: return launch_dma_cfg<192, 256, 96, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
-    case 5: return launch_dma_cfg<128, 128, 64, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
-    case 4: return launch_dma_cfg<256, 256, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+  if (m <= 16) return {0, 1};
+  if (g_tile_cfg >= 4) {
+    const int p = (epilogue == 0 && g_tile_parts > 0 && (k / 64) % g_tile_parts == 0) ? g_tile_parts : 1;
+    return {g_tile_cfg, p};
+  }
+  const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
+  const long long t64 = (long long)((m + 63) / 64) * ((n + 127) / 128);
+  if (m > 64 && t256 >= 160) {
+    // rounds of 256 workgroups times the time of a tile: a 192-row tile does 0.75 of the work
+    // of a 256-row one in 0.81 of the time
+    const long long t192 = (long long)((m + 255) / 256) * ((n + 191) / 192);
+    const long long cost256 = (t256 + 255) / 256 * 1000, cost192 = (t192 + 255) / 256 * 815;
+    return {cost192 < cost256 ? 6 : 4, 1};
+  }
+  if (m > 64 && (t128 >= 256 || m > 512)) return {5, epilogue ? 1 : k_slices(t128, k, 512, k / (4 * m))};
+  return {7, epilogue ? 1 : k_slices(t64, k, 256, k / (8 * m))};
+}
+
+template <int EPI, typename TO>
+static int launch_planned(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int m, int n, int k,
+                          hipStream_t s) {
+  const TilePlan plan = plan_tiles(m, n, k, EPI);
+  RB_REQUIRE(plan.cfg != 0, "rb_gemm_bf16: internal: M=%d N=%d K=%d is not a product for the tiled kernels", m, n, k);
+  RB_REQUIRE(plan.parts == 1 || workspace != nullptr, "rb_gemm_bf16: M=%d N=%d K=%d needs a workspace of %lld floats",
+             m, n, k, (long long)plan.parts * m * n);
+  const int p = plan.parts;
+  switch (plan.cfg) {
+    case 7: return launch_dma_cfg<128, 64, 32, 64, 64, 3, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
+    case 6: return launch_dma_cfg<192, 256, 96, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
+    case 5: return launch_dma_cfg<128, 128, 64, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
+    case 4: return launch_dma_cfg<256, 256, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
     case 3: return launch_tiled_cfg<256, 256, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
     case 2: return launch_tiled_cfg<256, 128, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
     default: return launch_tiled_cfg<128, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
   }
 }
 
-
 #define RB_BY_OUTPUT(FN, ...)                                                              \
   (epilogue == 0 ? (dtype_out == RB_F32 ? FN<0, float>(__VA_ARGS__) : FN<0, bf16_t>(__VA_ARGS__)) \
                  : (dtype_out == RB_F32 ? FN<1, float>(__VA_ARGS__) : FN<1, bf16_t>(__VA_ARGS__)))
 
-int gemm_tiled_launch(const bf16_t* x, const bf16_t* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
-                      hipStream_t s) {
-  return RB_BY_OUTPUT(launch_tiled, x, w, c, m, n, k, s);
+int gemm_tiled_parts(int m, int n, int k, int epilogue) {
+  const TilePlan plan = plan_tiles(m, n, k, epilogue);
+  return plan.cfg == 0 ? 0 : plan.parts;
 }
 
-int gemm_stream_parts(int m, int n, int k, int epilogue) { return stream_parts(m, n, k, epilogue); }
-
-int gemm_stream_launch(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int dtype_out, int epilogue,
-                       int m, int n, int k, hipStream_t s) {
-  return RB_BY_OUTPUT(launch_stream, x, w, c, workspace, m, n, k, s);
+int gemm_tiled_launch(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int dtype_out, int epilogue, int m,
+                      int n, int k, hipStream_t s) {
+  return RB_BY_OUTPUT(launch_planned, x, w, c, workspace, m, n, k, s);
 }
