@@ -48,7 +48,9 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_kernel(
   const int seq_start = cu_seqlens[b];
   const int q_len = cu_seqlens[b + 1] - seq_start;
   const int past = past_len[b];
-  const int wg_q0 = blockIdx.x * q_per_wg;
+  // the blocks of late queries have the most keys: they are started first, and the short ones
+  // fill the compute units that finish early
+  const int wg_q0 = (gridDim.x - 1 - blockIdx.x) * q_per_wg;
   if (wg_q0 >= q_len) return;
   const int q0 = wg_q0 + (wave / gw) * 32;
   const bool wave_on = q0 < q_len;
@@ -252,6 +254,9 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_kernel(
     }
 }
 
+static int g_prefill_waves = 0;
+extern "C" void rb_tune_prefill_waves(int nw) { g_prefill_waves = nw; }      // experiments only; 0 = built-in
+
 extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, const void* v_pages, void* out,
                                          const int32_t* cu_seqlens, const int32_t* past_len,
                                          const int32_t* block_table, int bt_stride, int n_seqs, int max_q_len,
@@ -267,7 +272,8 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
   const int gw = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
   // 8 waves (two per SIMD, which cover each other's softmax arithmetic) when the longest
   // sequence gives them all queries; 4 for short steps
-  const int nw = max_q_len > 32 * (4 / gw) ? 8 : 4;
+  int nw = max_q_len > 32 * (4 / gw) ? 8 : 4;
+  if (g_prefill_waves) nw = g_prefill_waves;
   const int q_per_wg = 32 * (nw / gw);
   dim3 grid((max_q_len + q_per_wg - 1) / q_per_wg, n_kv_heads * (group / gw), n_seqs);
   RB_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "rb_attention_prefill_bf16: batch or head count too large");
