@@ -96,6 +96,41 @@ def decode_run(engine, batch: int, steps: int, warmup: int, seed: int = 0, promp
     return dt, ctx_mean
 
 
+def probe(lib, device) -> dict:
+    """What this GPU reaches on a plain streaming read and on back-to-back bfloat16 MFMAs
+    (csrc/probe.hip): the practical ceilings beside the nominal peaks.  Timed with events on
+    the stream, so that launch overhead on the host does not count."""
+    import torch
+    sink = torch.zeros(1, dtype=torch.float32, device=device)
+
+    def timed(fn, reps: int) -> float:
+        fn(0)
+        _sync()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(reps):
+            fn(i)
+        end.record()
+        _sync()
+        return start.elapsed_time(end) * 1e-3 / reps
+
+    out = {}
+    pool = torch.empty((3 << 30) // 4, dtype=torch.int32, device=device).fill_(1)
+    for label, nbytes in (("read_1gb_gbps", 1 << 30), ("read_32mb_gbps", 32 << 20)):
+        copies = pool.numel() * 4 // nbytes
+        views = [pool[i * (nbytes // 4):(i + 1) * (nbytes // 4)] for i in range(copies)]
+        best = 0.0
+        for blocks in (1024, 2048, 4096, 8192):          # the best grid size counts
+            t = timed(lambda i: lib.probe_read(views[i % copies], sink, blocks), 12 if nbytes >= (1 << 30) else 96)
+            best = max(best, nbytes / t)
+        out[label] = round(best / 1e9, 1)
+    del pool
+    waves = 256 * 4 * 2
+    t = timed(lambda i: lib.probe_mfma(waves, 20000, sink), 2)
+    out["mfma_bf16_tflops"] = round(float(waves) * 20000 * 4 * 2 * 32 * 32 * 16 / t / 1e12, 1)
+    return out
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="bench")
     ap.add_argument("--gpus", type=int, default=1)
@@ -190,6 +225,8 @@ def main(argv=None) -> int:
             dtb, _ = decode_run(engine, b, steps, max(4, args.warmup // 2), seed=b, prompt_len=prompt_len)
             points[f"decode_b{b}"] = round(b * steps / dtb, 2)
         out["points"] = points
+        # the practical ceilings of this GPU, for reading the fractions above
+        out["probe"] = probe(engine.lib, engine.device)
 
     print(json.dumps(out))
     return 0

@@ -92,6 +92,12 @@ int rb_sample_workspace_bytes(int n_rows, int vocab);
 int rb_sample(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,
               int32_t* tokens, void* workspace, void* stream);
 
+// What the GPU reaches, measured the simplest way: rb_probe_read reads `bytes` bytes (a multiple of
+// 16) once with 16-byte loads from `blocks` workgroups of 256 lanes; rb_probe_mfma runs 4 * iters bfloat16 32x32x16 MFMAs in each of `waves`
+// waves (a multiple of 4).  `sink` is one float of device memory that is practically never written.
+int rb_probe_read(const void* p, long long bytes, int blocks, float* sink, void* stream);
+int rb_probe_mfma(int waves, int iters, float* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

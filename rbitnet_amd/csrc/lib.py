@@ -71,6 +71,8 @@ class Kernels:
             "rb_attention_decode_fused_bf16": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
                                                _P, _P],
             "rb_sample": [_P, _I, _I, _P, _P, _P, _P, _P],
+            "rb_probe_read": [_P, ctypes.c_longlong, _I, _P, _P],
+            "rb_probe_mfma": [_I, _I, _P, _P],
         }
         for name, args in sig.items():
             fn = getattr(L, name)
@@ -262,6 +264,22 @@ class Kernels:
             raise KernelError("sampling workspace too small")
         self._ok(self._lib.rb_sample(_ptr(logits), n, vocab, _ptr(temperature), _ptr(u), _ptr(tokens),
                                      _ptr(workspace), self._stream()))
+
+    # ------------------------------------------------------------------ probes
+    def probe_read(self, buf: torch.Tensor, sink: torch.Tensor, blocks: int = 2048) -> None:
+        """Reads every byte of `buf` once with `blocks` workgroups (see probe.hip)."""
+        _check(buf, "buf")
+        _check(sink, "sink", torch.float32)
+        nbytes = buf.numel() * buf.element_size()
+        if nbytes % 16 != 0 or buf.data_ptr() % 16 != 0:
+            raise KernelError("probe buffer must be 16-byte aligned and a multiple of 16 bytes long")
+        self._ok(self._lib.rb_probe_read(_ptr(buf), nbytes, int(blocks), _ptr(sink), self._stream()))
+
+    def probe_mfma(self, waves: int, iters: int, sink: torch.Tensor) -> float:
+        """Runs the MFMA loop; returns the floating-point operations it performs."""
+        _check(sink, "sink", torch.float32)
+        self._ok(self._lib.rb_probe_mfma(int(waves), int(iters), _ptr(sink), self._stream()))
+        return float(waves) * iters * 4 * 2 * 32 * 32 * 16
 
 
 _lock = threading.Lock()

@@ -508,3 +508,19 @@ def test_sample_frequencies_follow_softmax(lib):
     counts = torch.bincount(tokens.long().cpu(), minlength=vocab).double()
     want = torch.softmax(row.double() / temp, 0) * n
     assert float((counts - want).abs().max()) <= 2.0
+
+
+# ------------------------------------------------------------------------ probes
+def test_probes_run(lib):
+    """The streaming-read and MFMA probes of the benchmark launch, touch nothing but their
+    sink, and refuse a buffer they cannot read with 16-byte loads."""
+    from rbitnet_amd.errors import KernelError
+    sink = torch.zeros(1, device=DEV)
+    buf = torch.arange(1 << 20, dtype=torch.int32, device=DEV)
+    before = buf.clone()
+    lib.probe_read(buf, sink, 64)
+    assert lib.probe_mfma(8, 10, sink) == 8 * 10 * 4 * 2 * 32 * 32 * 16
+    torch.cuda.synchronize()
+    assert torch.equal(buf, before) and float(sink) == 0.0
+    with pytest.raises(KernelError):
+        lib.probe_read(buf[:3], sink)
