@@ -332,6 +332,16 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
 #pragma unroll
         for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[ks & 1][i], b[ks & 1][j], acc[i][j]);
     }
+    // the order the scheduler is asked to keep: the fragments of depth step ks + 1 are all
+    // requested before the MFMAs of step ks, which then cover the LDS latency
+    constexpr int KSTEPS = BK / 16;
+    __builtin_amdgcn_sched_group_barrier(0x100, TN + TM, 0);
+#pragma unroll
+    for (int ks = 0; ks + 1 < KSTEPS; ++ks) {
+      __builtin_amdgcn_sched_group_barrier(0x100, TN + TM, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, TN * TM, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TN * TM, 0);
   };
 
 #pragma unroll
