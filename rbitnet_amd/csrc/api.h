@@ -98,6 +98,18 @@ int rb_sample(const float* logits, int n_rows, int vocab, const float* temperatu
 int rb_probe_read(const void* p, long long bytes, int blocks, float* sink, void* stream);
 int rb_probe_mfma(int waves, int iters, float* sink, void* stream);
 
+// ---- experiment hooks: they override the built-in choice of kernel, tile or wave count for
+// measurements and for tests that must reach a kernel the dispatcher would not pick.  The
+// settings are process-wide and are read at every launch; 0 restores the built-in choice.
+void rb_tune(int stages, int rows_per_wave, int waves);         // skinny product
+void rb_tune_resident(int waves, int parts, int tiles);         // skinny product with resident tokens
+void rb_tune_use_resident(int on);                              // 0: never the resident variant
+void rb_tune_use_stream(int on);                                // 0: the skinny product up to 64 tokens
+void rb_tune_tiles(int cfg, int parts);                         // tiled product: tile configuration and K slices
+void rb_tune_prefill_waves(int waves);                          // prefill attention: 4 or 8
+void rb_tune_decode_mfma(int mode);                             // decode attention: 1 matrix cores, 2 vector units
+void rb_tune_decode_waves(int waves);                           // matrix-core decode attention: 4 or 8
+
 #ifdef __cplusplus
 }
 #endif
