@@ -103,7 +103,7 @@ int rb_probe_mfma(int waves, int iters, float* sink, void* stream);
 // settings are process-wide and are read at every launch; 0 restores the built-in choice.
 void rb_tune(int stages, int rows_per_wave, int waves);         // skinny product
 void rb_tune_resident(int waves, int parts, int tiles);         // skinny product with resident tokens
-void rb_tune_use_resident(int on);                              // 0: never the resident variant
+void rb_tune_use_resident(int on);                              // 0: never the resident variant, 2: also below 8192 rows
 void rb_tune_use_stream(int on);                                // 0: the skinny product up to 64 tokens
 void rb_tune_tiles(int cfg, int parts);                         // tiled product: tile configuration and K slices
 void rb_tune_prefill_waves(int waves);                          // prefill attention: 4 or 8

@@ -911,15 +911,16 @@ static int launch_decode_mfma_nw(const DecodeArgs& a, hipStream_t s) {
   return 0;
 }
 
-// 8 waves (8 pages at a time) while that still gives every workgroup a compute unit of its
-// own (a wave's page of V takes 16 KB of LDS at head size 128), else 4 waves and two
-// workgroups per compute unit.
+// 8 waves (8 pages at a time) for short contexts (one split) while that still gives every
+// workgroup a compute unit of its own (a wave's page of V takes 16 KB of LDS at head size
+// 128): the step is then bound by latency and fewer rounds of pages count.  Else 4 waves and
+// two workgroups per compute unit, which stream long contexts a little faster.
 static int g_decode_waves = 0;
 extern "C" void rb_tune_decode_waves(int nw) { g_decode_waves = nw; }      // experiments only; 0 = built-in
 template <int D, bool FUSED>
 static int launch_decode_mfma(const DecodeArgs& a, hipStream_t s) {
   const long long wgs = (long long)a.n_splits * a.n_kv * a.n_seqs;
-  const int nw = g_decode_waves ? g_decode_waves : (wgs <= 256 ? 8 : 4);
+  const int nw = g_decode_waves ? g_decode_waves : (wgs <= 256 && a.n_splits == 1 ? 8 : 4);
   return nw == 8 ? launch_decode_mfma_nw<D, 8, FUSED>(a, s) : launch_decode_mfma_nw<D, 4, FUSED>(a, s);
 }
 

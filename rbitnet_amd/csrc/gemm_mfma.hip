@@ -36,7 +36,7 @@ extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out
   int rc = 0;
   if (tiled_parts(m, n, k, epilogue) >= 1) {
     rc = gemm_tiled_launch(xa, wa, c, workspace, dtype_out, epilogue, m, n, k, s);
-  } else if (!(g_use_resident && m <= 16 && n > 8192 &&
+  } else if (!(g_use_resident && m <= 16 && (n > 8192 || g_use_resident == 2) &&
                gemm_resident_try(xa, wa, c, dtype_out, epilogue, m, n, k, s, &rc))) {
     rc = gemm_skinny_launch(xa, wa, c, dtype_out, epilogue, m, n, k, s);
   }

@@ -47,17 +47,23 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
     xrow[cb] = x + (size_t)(xok[cb] ? row : 0) * k;
   }
 
-  const int k_begin = wave * k_per_wave;
+  int k_begin = wave * k_per_wave;
   const int k_end = (k_begin + k_per_wave < k) ? k_begin + k_per_wave : k;
   if (FAST) {
     // K and every wave's range are multiples of 128: no bounds checks.  Rows beyond N or M
     // are read from row 0 instead and their results never stored.  U stages of 128 depth
     // values stay in flight: as soon as a stage has been multiplied, its registers are
     // loaded again with the stage U further on.
-    // The host chose the waves so that every wave has the same number of stages, a
-    // positive multiple of U: the loads below are unconditional, which lets the compiler
-    // count outstanding loads exactly and start multiplying when the oldest stage arrives.
-    const int stages = k_per_wave / 128;
+    // Every wave has at least one stage (the host launches no more waves than stages), and a
+    // wave's stage count is a multiple of U: the loads below are unconditional, which lets the
+    // compiler count outstanding loads exactly and start multiplying when the oldest stage
+    // arrives.  The K / 128 stages are dealt to the waves as evenly as they go: the first
+    // K / 128 % waves waves take one more (K = 11008 = 86 stages over 8 waves: six times 11,
+    // twice 10).
+    static_assert(U == 1, "uneven stage counts per wave need one stage in flight");
+    const int total = k / 128, base = total / n_waves, extra = total % n_waves;
+    const int stages = base + (wave < extra ? 1 : 0);
+    k_begin = 128 * (wave * base + (wave < extra ? wave : extra));
     Frag8 a[U][R][4], b[U][MB][4];
     auto load_stage = [&](int u, int st) {
       const int kk = k_begin + 128 * st + 8 * kq;
@@ -183,8 +189,8 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, void* c, int m, int n
   return 0;
 }
 
-// How K is dealt to the waves of a workgroup.  Fast path: K = 128 * T and the wave count
-// divides T.  Otherwise the checked path with up to 8 waves.  Measured on the Llama-3-8B
+// How K is dealt to the waves of a workgroup.  Fast path: K = 128 * T, the T stages dealt to
+// the waves as evenly as they go.  Otherwise the checked path with up to 8 waves.  Measured on the Llama-3-8B
 // products at M = 1..8: one stage in flight per wave (U = 1) is as fast as 2 or 4, and 4
 // waves beat 8 at K = 4096, 8 beat 4 at K = 14336.
 template <int MB, int R, int EPI, typename TO>
@@ -192,11 +198,10 @@ static int launch_skinny_u(const bf16_t* x, const bf16_t* w, void* c, int m, int
   constexpr int max_waves = (R * MB <= 4) ? 8 : (R * MB <= 8 ? 4 : 3);      // bounds the reduction buffer
   if (k % 128 == 0) {
     const int t = k / 128;
-    const int first_nw = (k >= 8192 || max_waves < 4) ? max_waves : 4;
-    for (int nw = g_tune_waves ? g_tune_waves : first_nw; nw >= 1; --nw) {
-      if (t % nw != 0) continue;
-      return launch_skinny<MB, R, 1, true, EPI, TO>(x, w, c, m, n, k, nw, k / nw, s);
-    }
+    int nw = g_tune_waves ? g_tune_waves : ((k >= 8192 || max_waves < 4) ? max_waves : 4);
+    if (nw > max_waves) nw = max_waves;
+    if (nw > t) nw = t;
+    return launch_skinny<MB, R, 1, true, EPI, TO>(x, w, c, m, n, k, nw, 0, s);
   }
   int n_waves = k / 256;
   if (n_waves < 1) n_waves = 1;
@@ -374,10 +379,12 @@ static int launch_resident(const bf16_t* x, const bf16_t* w, void* c, int m, int
   const int slices = k / (32 * XQ);
   const int n_waves = slices / parts;
   const int n_tiles = (n + 15) / 16;
-  // tiles per workgroup: as many as leave about one workgroup per compute unit (measured on
-  // the 28672 x 4096 and 128256 x 4096 products: 224 and 501 workgroups beat 448 and 1002)
-  int tiles = g_res_tiles ? g_res_tiles : 16;
-  while (!g_res_tiles && tiles > 2 && (long long)((n_tiles + tiles - 1) / tiles) * parts < 200) tiles >>= 1;
+  // tiles per workgroup: as many as give every compute unit one workgroup at most, but no more
+  // than 16 (measured: 22016 rows in 230 workgroups of 6 tiles take 35 us, in 344 of 4, which
+  // come in two rounds, 44 us; 12288 rows 20 us in 256 workgroups, 31 us in 384; the 128256
+  // rows of an output layer are as fast in 501 workgroups of 16 tiles as in 251 of 32)
+  int tiles = g_res_tiles ? g_res_tiles : (n_tiles + 255) / 256;
+  if (!g_res_tiles && tiles > 16) tiles = 16;
   if (EPI == 1 && (tiles & 1)) tiles += 1;
   const size_t lds = (size_t)2 * (n_waves > 1 ? n_waves - 1 : 0) * MB * 4 * 64 * sizeof(float);
   dim3 grid((n_tiles + tiles - 1) / tiles, parts);
