@@ -124,3 +124,21 @@ def test_uniform_is_keyed_by_seed_sequence_and_count():
     assert a == [uniform(0, 3, n) for n in range(50)]
     assert uniform(1, 3, 0) != a[0] and uniform(0, 4, 0) != a[0]
     assert abs(sum(uniform(7, i, 0) for i in range(2000)) / 2000 - 0.5) < 0.03
+
+
+def test_decode_attention_split_rule(monkeypatch):
+    """How many workgroups share the pages of one (sequence, kv head) in decode attention:
+    none up to 15 pages, two from 16 pages, four from 32 and so on to at most 16, and never more than gives
+    every compute unit about one workgroup; an environment variable overrides the rule."""
+    from rbitnet_amd.engine.context import decode_splits, split_bucket
+    monkeypatch.delenv("RBITNET_DECODE_SPLITS", raising=False)
+    assert [split_bucket(n) for n in (1, 64, 960, 961, 1024, 2047, 2049, 4096, 8192, 10 ** 6)] == \
+        [1, 1, 1, 2, 2, 4, 4, 8, 16, 16]
+    assert split_bucket(0) == 1
+    assert decode_splits(8, 8, split_bucket(600)) == 1
+    assert decode_splits(8, 8, split_bucket(4096)) == 4          # 256 // (8 * 8)
+    assert decode_splits(1, 8, split_bucket(4096)) == 8
+    assert decode_splits(64, 8, split_bucket(65536)) == 1
+    assert decode_splits(1, 1, 16) == 16
+    monkeypatch.setenv("RBITNET_DECODE_SPLITS", "3")
+    assert decode_splits(64, 8, 1) == 3
