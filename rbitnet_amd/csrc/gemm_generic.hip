@@ -1,5 +1,6 @@
 // C[M, N] = A[M, K] * W[N, K]^T for any sizes, float32 or bfloat16 storage, float32
-// multiply-add on the vector units (never a reduced-precision matrix mode).  This is the
+// multiply-add on the vector units or, for float32 operands with K % 16 == 0, the float32
+// MFMA (never a reduced-precision matrix mode).  This is the
 // whole float32 path's matrix product and the bfloat16 path's product for shapes the
 // matrix-core kernels refuse.
 //
@@ -128,6 +129,108 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
     }
 }
 
+// Float32 operands and more than 16 tokens with K a multiple of 16 (the float32 path's
+// prefill): the float32 MFMA (v_mfma_f32_32x32x2_f32: float32 inputs, float32 products and
+// sums; no reduced-precision mode).  128 x 128 tiles, 16 deep, one wave per 64 x 64 piece.  W
+// and the tokens are read with 16-byte loads along K and stored in LDS depth-major
+// ([k][row], rows padded by 4 floats), so that the 32 lanes that read one depth value of 32
+// rows hit 32 different banks; the next tile's loads are in flight in registers while the
+// current one is multiplied.  D layout of the MFMA: lane l holds column l % 32 (a token),
+// rows 8 * (i / 4) + 4 * (l / 32) + i % 4 (rows of W).
+typedef __attribute__((ext_vector_type(16))) float gf32x16_t;
+#define GM_T 128
+#define GM_K 16
+#define GM_LD (GM_T + 4)
+
+__global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                            float* __restrict__ c, int m, int n, int k) {
+  __shared__ float ws[2][GM_K][GM_LD];
+  __shared__ float xs[2][GM_K][GM_LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * GM_T, m0 = blockIdx.y * GM_T;
+  const int wn0 = (wave & 1) * 64, wm0 = (wave >> 1) * 64;
+  const int l32 = lane & 31, g = lane >> 5;
+
+  gf32x16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // staging: thread t loads, for q = t and t + 256, row q / 4 of the tile, depth values 4 (q % 4) .. + 3
+  const float* wp[2];
+  const float* xp[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = tid + 256 * i;
+    int wr = n0 + q / 4, xr = m0 + q / 4;
+    if (wr > n - 1) wr = n - 1;            // rows beyond the matrix: a valid row, never stored
+    if (xr > m - 1) xr = m - 1;
+    wp[i] = w + (size_t)wr * k + 4 * (q % 4);
+    xp[i] = x + (size_t)xr * k + 4 * (q % 4);
+  }
+  float4 wreg[2], xreg[2];
+  auto load_tile = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      wreg[i] = *reinterpret_cast<const float4*>(wp[i] + (size_t)kt * GM_K);
+      xreg[i] = *reinterpret_cast<const float4*>(xp[i] + (size_t)kt * GM_K);
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int q = tid + 256 * i;
+      const int row = q / 4, kk = 4 * (q % 4);
+      ws[buf][kk + 0][row] = wreg[i].x;
+      ws[buf][kk + 1][row] = wreg[i].y;
+      ws[buf][kk + 2][row] = wreg[i].z;
+      ws[buf][kk + 3][row] = wreg[i].w;
+      xs[buf][kk + 0][row] = xreg[i].x;
+      xs[buf][kk + 1][row] = xreg[i].y;
+      xs[buf][kk + 2][row] = xreg[i].z;
+      xs[buf][kk + 3][row] = xreg[i].w;
+    }
+  };
+  const int k_tiles = k / GM_K;
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < k_tiles) load_tile(kt + 1);
+#pragma unroll
+    for (int ks = 0; ks < GM_K / 2; ++ks) {
+      float a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = ws[buf][2 * ks + g][wn0 + 32 * i + l32];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) b[j] = xs[buf][2 * ks + g][wm0 + 32 * j + l32];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < k_tiles) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int mm = m0 + wm0 + 32 * j + l32;
+      if (mm >= m) continue;
+      float* dst = c + (size_t)mm * n;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int nn = n0 + wn0 + 32 * i + 8 * (e / 4) + 4 * g + (e % 4);
+        if (nn < n) dst[nn] = acc[i][j][e];
+      }
+    }
+}
+
 extern "C" int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dtype_out, int m, int n,
                                int k, void* stream) {
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_generic: bad sizes M=%d N=%d K=%d", m, n, k);
@@ -140,6 +243,13 @@ extern "C" int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_
     if (m <= 4) gemm_f32_skinny_kernel<4><<<blocks, 256, 0, s>>>(af, wf, (float*)c, m, n, k);
     else if (m <= 8) gemm_f32_skinny_kernel<8><<<blocks, 256, 0, s>>>(af, wf, (float*)c, m, n, k);
     else gemm_f32_skinny_kernel<16><<<blocks, 256, 0, s>>>(af, wf, (float*)c, m, n, k);
+    RB_LAUNCH_CHECK();
+    return 0;
+  }
+  if (dtype_in == RB_F32 && dtype_out == RB_F32 && m > 16 && k % GM_K == 0) {
+    dim3 tiles((n + GM_T - 1) / GM_T, (m + GM_T - 1) / GM_T);
+    RB_REQUIRE(tiles.y <= 65535, "rb_gemm_generic: M=%d too large for one launch", m);
+    gemm_f32_mfma_kernel<<<tiles, 256, 0, s>>>((const float*)a, (const float*)w, (float*)c, m, n, k);
     RB_LAUNCH_CHECK();
     return 0;
   }

@@ -45,7 +45,8 @@ def test_reference_matvec_vectors(lib):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 130, 67), (65, 64, 16), (130, 200, 333), (1, 130, 64), (8, 1000, 2052),
-                                   (16, 33, 4096), (5, 300, 1028), (4, 17, 4), (17, 50, 64)])
+                                   (16, 33, 4096), (5, 300, 1028), (4, 17, 4), (17, 50, 64), (17, 50, 60), (300, 200, 336),
+                                   (129, 1000, 16), (2048, 130, 256)])
 def test_gemm_generic_f32(lib, m, n, k):
     g = torch.Generator().manual_seed(m * 1000 + n)
     a = torch.randn(m, k, generator=g)
