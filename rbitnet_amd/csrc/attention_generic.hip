@@ -1,6 +1,10 @@
 // Causal attention of each token over its sequence's paged cache: any even head_dim up to
 // 256, any number of heads and groups, float32 or bfloat16 storage, float32 arithmetic
-// throughout (scores, softmax, weighted sum).  One wave per (token, query head).
+// throughout (scores, softmax, weighted sum).  One workgroup per (token, query head): one wave
+// when the step has many tokens, up to 8 waves that share the pages of the context and merge
+// their running softmax states through LDS when it has few (a decode step of 8 sequences and
+// 32 heads would otherwise leave three quarters of the GPU idle, each wave walking its whole
+// context alone).
 //
 // Reference: kv head = q head / (Hq / Hk); s[p] = (q . K[p]) * scale for p <= pos;
 // softmax with the maximum subtracted; out = sum_p s[p] V[p]  (llama/model.rs:260-289,
@@ -13,24 +17,30 @@
 
 #define AG_MAX_D 256
 
+#define AG_MAX_WAVES 8
+
 template <typename T>
-__global__ __launch_bounds__(RB_WAVE) void attention_generic_kernel(
+__global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages, T* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
     const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, int head_dim, float scale,
     int window) {
   __shared__ float qs[AG_MAX_D];
-  __shared__ float ps[RB_PAGE];
+  __shared__ float ps_all[AG_MAX_WAVES][RB_PAGE];
+  __shared__ float red_m[AG_MAX_WAVES], red_l[AG_MAX_WAVES];
+  __shared__ float red_acc[AG_MAX_WAVES][AG_MAX_D];
   const int t = blockIdx.x;
   const int h = blockIdx.y;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & (RB_WAVE - 1);
+  const int wave = threadIdx.x / RB_WAVE, n_waves = blockDim.x / RB_WAVE;
+  float* ps = ps_all[wave];
   const int pos = tok_pos[t];
   const int kvh = h / (n_heads / n_kv);
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int32_t* pages = block_table + (size_t)tok_seq[t] * bt_stride;
 
   const T* qrow = q + ((size_t)t * n_heads + h) * head_dim;
-  for (int d = lane; d < head_dim; d += RB_WAVE) qs[d] = Num<T>::load(qrow + d);
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) qs[d] = Num<T>::load(qrow + d);
   __syncthreads();
 
   float m_run = -INFINITY, l_run = 0.f;
@@ -38,7 +48,7 @@ __global__ __launch_bounds__(RB_WAVE) void attention_generic_kernel(
 #pragma unroll
   for (int i = 0; i < AG_MAX_D / RB_WAVE; ++i) acc[i] = 0.f;
 
-  for (int pg = lo / RB_PAGE; pg <= pos / RB_PAGE; ++pg) {
+  for (int pg = lo / RB_PAGE + wave; pg <= pos / RB_PAGE; pg += n_waves) {
     const size_t base = ((size_t)pages[pg] * n_kv + kvh) * RB_PAGE * head_dim;
     const int p = pg * RB_PAGE + lane;
     float s = -INFINITY;
@@ -53,9 +63,9 @@ __global__ __launch_bounds__(RB_WAVE) void attention_generic_kernel(
     const float corr = (m_run == -INFINITY) ? 0.f : expf(m_run - m_new);
     l_run = l_run * corr + wave_sum(pexp);
     m_run = m_new;
-    __syncthreads();
+    // ps belongs to this wave alone; a wave's LDS accesses complete in order
     ps[lane] = pexp;
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();
     const int j_lo = (pg * RB_PAGE < lo) ? lo - pg * RB_PAGE : 0;
     const int j_hi = (pg * RB_PAGE + RB_PAGE - 1 > pos) ? pos - pg * RB_PAGE : RB_PAGE - 1;
 #pragma unroll
@@ -66,6 +76,34 @@ __global__ __launch_bounds__(RB_WAVE) void attention_generic_kernel(
         const T* vcol = v_pages + base + d;
         for (int j = j_lo; j <= j_hi; ++j) a = fmaf(ps[j], Num<T>::load(vcol + (size_t)j * head_dim), a);
         acc[i] = a;
+      }
+    }
+  }
+  // ---- the waves' states into one (a wave without pages holds m = -inf, l = 0, acc = 0)
+  if (n_waves > 1) {
+    if (lane == 0) {
+      red_m[wave] = m_run;
+      red_l[wave] = l_run;
+    }
+#pragma unroll
+    for (int i = 0; i < AG_MAX_D / RB_WAVE; ++i) {
+      const int d = lane + i * RB_WAVE;
+      if (d < head_dim) red_acc[wave][d] = acc[i];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float mx = red_m[0];
+    for (int w = 1; w < n_waves; ++w) mx = fmaxf(mx, red_m[w]);
+    l_run = 0.f;
+#pragma unroll
+    for (int i = 0; i < AG_MAX_D / RB_WAVE; ++i) acc[i] = 0.f;
+    for (int w = 0; w < n_waves; ++w) {
+      const float f = (red_m[w] == -INFINITY) ? 0.f : expf(red_m[w] - mx);
+      l_run += red_l[w] * f;
+#pragma unroll
+      for (int i = 0; i < AG_MAX_D / RB_WAVE; ++i) {
+        const int d = lane + i * RB_WAVE;
+        if (d < head_dim) acc[i] += red_acc[w][d] * f;
       }
     }
   }
@@ -91,13 +129,17 @@ extern "C" int rb_attention_generic(const void* q, const void* k_pages, const vo
   if (n_tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(n_tokens, n_heads);
+  // waves per (token, head): enough to give every SIMD of the GPU a wave, at most 8
+  int n_waves = 1;
+  while (n_waves < AG_MAX_WAVES && (long long)n_tokens * n_heads * n_waves < 1024) n_waves *= 2;
+  const int threads = RB_WAVE * n_waves;
   if (dtype == RB_F32)
-    attention_generic_kernel<float><<<grid, RB_WAVE, 0, s>>>((const float*)q, (const float*)k_pages,
+    attention_generic_kernel<float><<<grid, threads, 0, s>>>((const float*)q, (const float*)k_pages,
                                                             (const float*)v_pages, (float*)out, tok_pos, tok_seq,
                                                             block_table, bt_stride, n_heads, n_kv_heads, head_dim,
                                                             scale, window);
   else if (dtype == RB_BF16)
-    attention_generic_kernel<bf16_t><<<grid, RB_WAVE, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages,
+    attention_generic_kernel<bf16_t><<<grid, threads, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages,
                                                              (const bf16_t*)v_pages, (bf16_t*)out, tok_pos,
                                                              tok_seq, block_table, bt_stride, n_heads, n_kv_heads,
                                                              head_dim, scale, window);
