@@ -55,6 +55,20 @@ long long rb_gemm_workspace_floats(int m, int n, int k, int epilogue);
 int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
                  float* workspace, void* stream);
 
+// The same product for 1..16 tokens with what stands before and after it in a decode step folded
+// in, so that no kernel runs between the products.  rb_gemm_bf16_few_ok: whether it takes these
+// sizes (few tokens, and no tiled kernel would).
+//   a: bfloat16 rows of K values; row i of the product is row rows[i] (row i without rows).
+//   squares_in (may be null): float32 [*, ceil(K / 16)], rows as in a.  Then a holds float32 rows
+//     times a norm's gain and squares_in their sums of squares over every 16 columns, and the
+//     product is multiplied by 1 / sqrt(sum of them / K + eps): the RMS norm's factor.
+//   epilogue 0, 1: as above.  2: C (float32) += product.  3: as 2, and for the norm that follows
+//     gained [M, N] = bf16(C * gain), squares_out [M, ceil(N / 16)] = sums of C^2 over 16 columns.
+int rb_gemm_bf16_few_ok(int m, int n, int k);
+int rb_gemm_bf16_few(const void* a, const float* squares_in, float eps, const int32_t* rows, const void* w, void* c,
+                     int dtype_out, int epilogue, const float* gain, void* gained, float* squares_out, int m, int n,
+                     int k, void* stream);
+
 // Causal attention of every token over its sequence's cache (keys 0..pos, or the last
 // `window` of them), any head_dim that is even and at most 256.
 //   q [T, Hq, D], out [T, Hq * D], both of dtype; pages as in rb_rope_kv_write.

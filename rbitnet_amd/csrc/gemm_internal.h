@@ -5,13 +5,36 @@
 
 #include "mfma.h"
 
-// at most 64 tokens, any K % 8 == 0: W streamed straight into MFMA operands (gemm_skinny.hip)
-int gemm_skinny_launch(const bf16_t* x, const bf16_t* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
-                       hipStream_t s);
+// The token operand of a product: bfloat16 rows of K values; row i of the product is row
+// rows[i] of x (row i without rows).  With squares ([*, ceil(K / 16)], rows as in x) the rows are
+// a float32 row times a norm's gain and squares holds that float32 row's sums of squares, one
+// for every 16 columns: the product is multiplied by 1 / sqrt(their sum / K + eps), which makes
+// it the product of the RMS-normalised row.
+struct GemmTokens {
+  const bf16_t* x;
+  const float* squares;
+  float eps;
+  const int32_t* rows;
+};
+
+// What becomes of the sums.  epilogue 0: C = sums; 1: the gated pair; 2: C (float32) += sums;
+// 3: as 2, and for the norm that follows gained [M, N] = bf16(C * gain) and
+// squares [M, ceil(N / 16)] = the sums of C^2 over every 16 columns.
+struct GemmAfter {
+  int epilogue;
+  const float* gain;
+  bf16_t* gained;
+  float* squares;
+};
+
+// at most 64 tokens, any K % 8 == 0: W streamed straight into MFMA operands (gemm_skinny.hip);
+// prepared tokens and epilogues 2 and 3: at most 16 tokens
+int gemm_skinny_launch(const GemmTokens& x, const bf16_t* w, void* c, int dtype_out, const GemmAfter& after, int m,
+                       int n, int k, hipStream_t s);
 // at most 16 tokens kept in registers while a workgroup walks several row tiles; false: these
 // sizes are not for it and nothing was launched
-bool gemm_resident_try(const bf16_t* x, const bf16_t* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
-                       hipStream_t s, int* rc);
+bool gemm_resident_try(const GemmTokens& x, const bf16_t* w, void* c, int dtype_out, const GemmAfter& after, int m,
+                       int n, int k, hipStream_t s, int* rc);
 // more than 16 tokens (more than 64 when K is no multiple of 64): tiles through LDS
 // (gemm_tiled.hip).  gemm_tiled_parts: 0 when these sizes are not for it, else the number of K
 // slices it will use; more than 1 needs parts * m * n floats of workspace.

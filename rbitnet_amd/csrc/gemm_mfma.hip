@@ -22,6 +22,16 @@ extern "C" long long rb_gemm_workspace_floats(int m, int n, int k, int epilogue)
   return p > 1 ? (long long)p * m * n : 0;
 }
 
+// products that no tiled kernel takes: the two kernels of gemm_skinny.hip
+static int launch_few_tokens(const GemmTokens& x, const bf16_t* w, void* c, int dtype_out, const GemmAfter& after,
+                             int m, int n, int k, hipStream_t s) {
+  int rc = 0;
+  if (g_use_resident && m <= 16 && (n > 8192 || g_use_resident == 2) &&
+      gemm_resident_try(x, w, c, dtype_out, after, m, n, k, s, &rc))
+    return rc;
+  return gemm_skinny_launch(x, w, c, dtype_out, after, m, n, k, s);
+}
+
 extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out, int epilogue, int m, int n,
                             int k, float* workspace, void* stream) {
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_bf16: bad sizes M=%d N=%d K=%d", m, n, k);
@@ -36,10 +46,35 @@ extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out
   int rc = 0;
   if (tiled_parts(m, n, k, epilogue) >= 1) {
     rc = gemm_tiled_launch(xa, wa, c, workspace, dtype_out, epilogue, m, n, k, s);
-  } else if (!(g_use_resident && m <= 16 && (n > 8192 || g_use_resident == 2) &&
-               gemm_resident_try(xa, wa, c, dtype_out, epilogue, m, n, k, s, &rc))) {
-    rc = gemm_skinny_launch(xa, wa, c, dtype_out, epilogue, m, n, k, s);
+  } else {
+    const GemmTokens x = {xa, nullptr, 0.f, nullptr};
+    const GemmAfter after = {epilogue, nullptr, nullptr, nullptr};
+    rc = launch_few_tokens(x, wa, c, dtype_out, after, m, n, k, s);
   }
+  if (rc) return rc;
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int rb_gemm_bf16_few_ok(int m, int n, int k) {
+  return m >= 1 && m <= 16 && n > 0 && k > 0 && k % 8 == 0 && tiled_parts(m, n, k, 0) == 0;
+}
+
+extern "C" int rb_gemm_bf16_few(const void* a, const float* squares_in, float eps, const int32_t* rows, const void* w,
+                                void* c, int dtype_out, int epilogue, const float* gain, void* gained,
+                                float* squares_out, int m, int n, int k, void* stream) {
+  RB_REQUIRE(rb_gemm_bf16_few_ok(m, n, k), "rb_gemm_bf16_few: M=%d N=%d K=%d is not for it (1..16 tokens, K %% 8 == 0)",
+             m, n, k);
+  RB_REQUIRE(epilogue >= 0 && epilogue <= 3, "rb_gemm_bf16_few: unknown epilogue %d", epilogue);
+  RB_REQUIRE(epilogue != 1 || n % 32 == 0, "rb_gemm_bf16_few: gated epilogue needs N=%d to be a multiple of 32", n);
+  RB_REQUIRE(dtype_out == RB_F32 || (dtype_out == RB_BF16 && epilogue <= 1),
+             "rb_gemm_bf16_few: output dtype %d with epilogue %d", dtype_out, epilogue);
+  RB_REQUIRE(!squares_in || epilogue <= 1, "rb_gemm_bf16_few: prepared rows go with epilogues 0 and 1, not %d", epilogue);
+  RB_REQUIRE(epilogue != 3 || (gain && gained && squares_out),
+             "rb_gemm_bf16_few: epilogue 3 needs the gain and room for the prepared rows");
+  const GemmTokens x = {(const bf16_t*)a, squares_in, eps, rows};
+  const GemmAfter after = {epilogue, gain, (bf16_t*)gained, squares_out};
+  const int rc = launch_few_tokens(x, (const bf16_t*)w, c, dtype_out, after, m, n, k, (hipStream_t)stream);
   if (rc) return rc;
   RB_LAUNCH_CHECK();
   return 0;

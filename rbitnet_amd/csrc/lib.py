@@ -65,6 +65,8 @@ class Kernels:
             "rb_swiglu": [_P, _P, _I, _I, _I, _P],
             "rb_gemm_generic": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
             "rb_gemm_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P],
+            "rb_gemm_bf16_few": [_P, _P, _F, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _P],
+            "rb_gemm_bf16_few_ok": [_I, _I, _I],
             "rb_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_prefill_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_decode_bf16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
@@ -170,6 +172,39 @@ class Kernels:
         workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need else None
         self._ok(self._lib.rb_gemm_bf16(_ptr(a), _ptr(w), _ptr(c), dtype_code(c.dtype), int(epilogue), m, n, k,
                                         _ptr(workspace), self._stream()))
+
+    def gemm_bf16_few_ok(self, m: int, n: int, k: int) -> bool:
+        """Whether gemm_bf16_few takes these sizes (1..16 tokens)."""
+        return bool(self._lib.rb_gemm_bf16_few_ok(int(m), int(n), int(k)))
+
+    def gemm_bf16_few(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = 0,
+                      squares: Optional[torch.Tensor] = None, eps: float = 0.0, rows: Optional[torch.Tensor] = None,
+                      gain: Optional[torch.Tensor] = None, gained: Optional[torch.Tensor] = None,
+                      squares_out: Optional[torch.Tensor] = None) -> None:
+        """The product of 1..16 tokens with its neighbours folded in.
+        squares [*, ceil(K / 16)]: a holds rows times a norm's gain and squares the sums of squares
+        of the rows themselves; the product is scaled to that of the RMS-normalised rows (eps).
+        rows: the tokens are these rows of a (and of squares).
+        epilogue 2: c (float32) += product.  epilogue 3: the same, and gained [M, N] =
+        bf16(c * gain), squares_out [M, ceil(N / 16)] = sums of c^2, for the norm that follows."""
+        n, k = w.shape
+        _check(a, "a", torch.bfloat16)
+        if a.dim() != 2 or a.shape[1] != k:
+            raise KernelError(f"a must have rows of {k} values, found {tuple(a.shape)}")
+        m = a.shape[0] if rows is None else rows.shape[0]
+        if rows is not None:
+            _check(rows, "rows", torch.int32, (m,))
+        if squares is not None:
+            _check(squares, "squares", torch.float32, (a.shape[0], (k + 15) // 16))
+        _check(w, "w", torch.bfloat16, (n, k))
+        _check(c, "c", torch.float32 if epilogue >= 2 else None, (m, n // 2 if epilogue == 1 else n))
+        if epilogue == 3:
+            _check(gain, "gain", torch.float32, (n,))
+            _check(gained, "gained", torch.bfloat16, (m, n))
+            _check(squares_out, "squares_out", torch.float32, (m, (n + 15) // 16))
+        self._ok(self._lib.rb_gemm_bf16_few(_ptr(a), _ptr(squares), float(eps), _ptr(rows), _ptr(w), _ptr(c),
+                                            dtype_code(c.dtype), int(epilogue), _ptr(gain), _ptr(gained),
+                                            _ptr(squares_out), m, n, k, self._stream()))
 
     def attention_generic(self, q, k_pages, v_pages, out, tok_pos, tok_seq, block_table, n_heads, n_kv, head_dim,
                           scale, window) -> None:

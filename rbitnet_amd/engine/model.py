@@ -16,6 +16,7 @@ import torch
 from ..config.spec import ModelSpec
 from ..errors import ConfigError
 from ..parts.base import BuildEnv, CacheRequest, TensorSpec, build_part
+from ..parts.block import normed_for
 from ..parts.linear import linear
 
 
@@ -63,6 +64,8 @@ def expected_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:
 
 
 class Model:
+    takes_gained_rows = True      # the output product takes what the last product left for the final norm
+
     def __init__(self, spec: ModelSpec, dtype: torch.dtype, device, lib, generic_only: bool = False):
         if dtype not in (torch.float32, torch.bfloat16):
             raise ConfigError(f"compute dtype must be float32 or bfloat16, not {dtype}")
@@ -168,7 +171,15 @@ class Model:
         x = torch.empty((ctx.n_tokens, self.spec.hidden_size), dtype=torch.float32, device=self.device)
         self.lib.embed_gather(self.embedding, ctx.token_ids, x)
         pending = None
-        for place, i in enumerate(self.spec.schedule):
-            pending = self.blocks[i].forward(x, pending, ctx, cache.view(place, ctx.block_tables))
-        xn = self.final_norm.forward(x, pending, rows)
+        schedule = self.spec.schedule
+        for place, i in enumerate(schedule):
+            block = self.blocks[i]
+            view = cache.view(place, ctx.block_tables)
+            if getattr(block, "takes_next_norm", False):
+                after = self.blocks[schedule[place + 1]] if place + 1 < len(schedule) else None
+                next_norm = self.final_norm if after is None else getattr(after, "first_norm", None)
+                pending = block.forward(x, pending, ctx, view, next_norm=next_norm)
+            else:
+                pending = block.forward(x, pending, ctx, view)
+        xn = normed_for(self, self.final_norm, x, pending, rows)
         return linear(self.lib, xn, self.head, torch.float32)

@@ -18,6 +18,11 @@ Interface of a mixer:
   tensor_specs() / load(tensors)
   cache_request() -> CacheRequest or None
   forward(h [T, E] compute dtype, ctx, view) -> float32 [T, E]
+Two things a mixer may say of itself (this one does both):
+  adds_to_stream: forward also takes stream=x (float32 [T, E], the residual stream) and
+  next_norm (the norm that follows) and may add its result to the stream itself; it then returns
+  None, or the GainedRows that its last product left for next_norm;
+  takes_gained_rows: h may be such GainedRows instead of a tensor.
 """
 from __future__ import annotations
 
@@ -27,7 +32,7 @@ import torch
 
 from ..errors import ConfigError, KernelError
 from .base import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register_mixer
-from .linear import linear
+from .linear import linear, linear_to_stream
 
 DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight"}
 _MATRIX_CORE_HEAD_DIMS = (64, 128)
@@ -36,6 +41,8 @@ _DECODE_GROUPS = tuple(range(1, 17))    # query heads per kv head the decode ker
 
 class Attention(Part):
     graph_safe = True
+    takes_gained_rows = True
+    adds_to_stream = True
 
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env
@@ -83,7 +90,7 @@ class Attention(Part):
                             window=None if self.window is None else int(self.window))
 
     # ------------------------------------------------------------------ forward
-    def forward(self, h: torch.Tensor, ctx, view) -> torch.Tensor:
+    def forward(self, h, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None):
         lib = self.env.lib
         t = h.shape[0]
         hq, hk, d = self.n_heads, self.n_kv, self.head_dim
@@ -102,7 +109,7 @@ class Attention(Part):
             n_splits, workspace = ctx.decode_workspace(hq, d, hk)
             lib.attention_decode_fused_bf16(qkv, cos, sin, style, view.k_pages, view.v_pages, attn, ctx.tok_pos, bt,
                                             hq, hk, d, self.scale, window, n_splits, workspace)
-            return linear(lib, attn, self.w_o, torch.float32)
+            return linear_to_stream(lib, attn, self.w_o, stream, next_norm)
         q = torch.empty((t, hq, d), dtype=self.env.dtype, device=h.device)
         if owns:
             self.position.encode_and_store(qkv, q, view.k_pages, view.v_pages, ctx, bt, hq, hk, d)
@@ -118,7 +125,7 @@ class Attention(Part):
         else:
             lib.attention_generic(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, bt, hq, hk, d,
                                   self.scale, window)
-        return linear(lib, attn, self.w_o, torch.float32)
+        return linear_to_stream(lib, attn, self.w_o, stream, next_norm)
 
 
 register_mixer("attention", Attention)

@@ -7,7 +7,8 @@ product's epilogue, on the generic path by a small kernel on its float32 result.
 
 Parameters: intermediate_size, activation ("silu"), names.
 Interface of a feed-forward: tensor_specs() / load(tensors) / forward(h [T, E], ctx) ->
-float32 [T, E].
+float32 [T, E].  It may say `takes_gained_rows` and `adds_to_stream` of itself as a mixer
+may (this one does both).
 """
 from __future__ import annotations
 
@@ -17,13 +18,15 @@ import torch
 
 from ..errors import ConfigError
 from .base import BuildEnv, Part, TensorSpec, register_feed_forward
-from .linear import can_fuse_gate, gated_linear, linear, pack_gate_up
+from .linear import can_fuse_gate, gated_linear, linear_to_stream, pack_gate_up
 
 DEFAULT_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
 
 
 class SwiGLU(Part):
     graph_safe = True
+    takes_gained_rows = True
+    adds_to_stream = True
 
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env
@@ -45,10 +48,10 @@ class SwiGLU(Part):
         self.w_gate_up = pack_gate_up(tensors[self.names["gate"]], tensors[self.names["up"]], self.fused)
         self.w_down = tensors[self.names["down"]].contiguous()
 
-    def forward(self, h: torch.Tensor, ctx=None) -> torch.Tensor:
+    def forward(self, h, ctx=None, stream: Optional[torch.Tensor] = None, next_norm=None):
         lib = self.env.lib
         t = gated_linear(lib, h, self.w_gate_up, self.ff, self.fused)
-        return linear(lib, t, self.w_down, torch.float32)
+        return linear_to_stream(lib, t, self.w_down, stream, next_norm)
 
 
 register_feed_forward("swiglu", SwiGLU)

@@ -4,12 +4,20 @@ matvec loops read it (crates/bitnet-core/src/llama/model.rs:67-91).  No biases.
 float32 operands run on the vector units in true 32-bit arithmetic; bfloat16
 operands run on the matrix cores with float32 accumulation when the inner size
 is a multiple of 8 (16-byte rows), else through the same generic kernel.
+
+A product's result may be meant for the residual stream (`linear_to_stream`), and the tokens
+may come as `GainedRows`, which such a product left for the norm after it.  With few tokens
+on the matrix cores the products do the sums and the norms themselves and no kernel runs
+between them; otherwise the caller is left with the sum and the rows are normalised first.
 """
 from __future__ import annotations
+
+from typing import Optional
 
 import torch
 
 from ..errors import KernelError
+from .norm import GainedRows
 
 GATE_BLOCK = 16     # rows per block when gate and up rows are interleaved for the fused epilogue
 
@@ -18,13 +26,28 @@ def uses_matrix_cores(dtype: torch.dtype, k: int) -> bool:
     return dtype == torch.bfloat16 and k % 8 == 0
 
 
-def linear(lib, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+def _few(lib, x, w: torch.Tensor) -> bool:
+    """Whether the kernel for a few tokens, which folds its neighbours in, takes this product."""
+    m, k = x.shape
+    return uses_matrix_cores(x.dtype, k) and lib.gemm_bf16_few_ok(m, w.shape[0], k)
+
+
+def _from_gained(lib, x: GainedRows, w: torch.Tensor, out: torch.Tensor, epilogue: int) -> None:
+    lib.gemm_bf16_few(x.gained, w, out, epilogue, squares=x.squares, eps=x.eps, rows=x.rows)
+
+
+def linear(lib, x, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     """[M, K] x [N, K]^T -> [M, N] in `out_dtype`."""
     m, k = x.shape
     n = w.shape[0]
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     if m == 0:
         return out
+    if isinstance(x, GainedRows):
+        if _few(lib, x, w):
+            _from_gained(lib, x, w, out, 0)
+            return out
+        x = x.tensor()
     if uses_matrix_cores(x.dtype, k):
         lib.gemm_bf16(x, w, out, 0)
     else:
@@ -32,6 +55,22 @@ def linear(lib, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> tor
             raise KernelError("a float32 product has a float32 result")
         lib.gemm_generic(x, w, out)
     return out
+
+
+def linear_to_stream(lib, x: torch.Tensor, w: torch.Tensor, stream: Optional[torch.Tensor], next_norm=None):
+    """x W^T as a float32 term of the residual stream [M, N].  Without a stream, or where the
+    product cannot add to it itself, the term comes back.  Otherwise it is added, and what comes
+    back is None, or, if the norm that follows folds into products, the `GainedRows` for it."""
+    if stream is None or x.shape[0] == 0 or not _few(lib, x, w):
+        return linear(lib, x, w, torch.float32)
+    if next_norm is None or not getattr(next_norm, "folds_into_products", False):
+        lib.gemm_bf16_few(x, w, stream, 2)
+        return None
+    m, n = stream.shape
+    gained = torch.empty((m, n), dtype=torch.bfloat16, device=stream.device)
+    squares = torch.empty((m, (n + 15) // 16), dtype=torch.float32, device=stream.device)
+    lib.gemm_bf16_few(x, w, stream, 3, gain=next_norm.weight, gained=gained, squares_out=squares)
+    return GainedRows(next_norm, stream, gained, squares)
 
 
 def can_fuse_gate(dtype: torch.dtype, k: int, ff: int) -> bool:
@@ -51,12 +90,17 @@ def pack_gate_up(gate: torch.Tensor, up: torch.Tensor, fused: bool) -> torch.Ten
     return torch.stack([g, u], dim=1).reshape(2 * ff, k).contiguous()
 
 
-def gated_linear(lib, x: torch.Tensor, w_packed: torch.Tensor, ff: int, fused: bool) -> torch.Tensor:
+def gated_linear(lib, x, w_packed: torch.Tensor, ff: int, fused: bool) -> torch.Tensor:
     """silu(x Wg^T) * (x Wu^T) -> [M, ff] in x's dtype."""
     m = x.shape[0]
     out = torch.empty((m, ff), dtype=x.dtype, device=x.device)
     if m == 0:
         return out
+    if isinstance(x, GainedRows):
+        if fused and _few(lib, x, w_packed):
+            _from_gained(lib, x, w_packed, out, 1)
+            return out
+        x = x.tensor()
     if fused:
         lib.gemm_bf16(x, w_packed, out, 1)
     else:

@@ -10,6 +10,11 @@ Interface of a norm: forward(x, delta=None, rows=None) -> h
   x      float32 [T, E], the residual stream; updated in place when delta is given
   delta  float32 [T, E] or None
   rows   int32 [R] or None: normalise only these rows (x is then left as it is)
+
+A norm that says `folds_into_products` (with weight, eps and size as here) lets the product
+before it and the product after it do its work when a step has few tokens: the first, which
+adds to the stream, also leaves bf16(x * gain) and the sums of x^2 (`GainedRows`); the second
+takes these as its tokens and multiplies its result by 1 / sqrt(mean(x^2) + eps).
 """
 from __future__ import annotations
 
@@ -20,8 +25,39 @@ import torch
 from .base import BuildEnv, Part, TensorSpec, register_norm
 
 
+class GainedRows:
+    """Rows of the float32 stream `x` (all, or those `rows` names) as a product left them for
+    `norm`: gained [T, E] = bf16(x * gain) and squares [T, ceil(E / 16)], the sums of x^2 over
+    every 16 columns.  What is left of the norm is one factor per row.  `linear` takes them as
+    tokens; tensor() normalises the rows with the norm's own kernel instead.  shape, dtype and
+    device are those of the normalised rows."""
+
+    def __init__(self, norm: "RMSNorm", x: torch.Tensor, gained: torch.Tensor, squares: torch.Tensor,
+                 rows: Optional[torch.Tensor] = None):
+        self.norm = norm
+        self.x = x
+        self.gained = gained
+        self.squares = squares
+        self.rows = rows
+        self.eps = norm.eps
+        self.shape = (x.shape[0] if rows is None else rows.shape[0], norm.size)
+        self.dtype = norm.env.dtype
+        self.device = x.device
+
+    def select(self, rows: Optional[torch.Tensor]) -> "GainedRows":
+        if rows is None:
+            return self
+        if self.rows is not None:
+            raise ValueError("rows were chosen already")
+        return GainedRows(self.norm, self.x, self.gained, self.squares, rows)
+
+    def tensor(self) -> torch.Tensor:
+        return self.norm.forward(self.x, None, self.rows)
+
+
 class RMSNorm(Part):
     graph_safe = True
+    folds_into_products = True
 
     def __init__(self, params: Dict, env: BuildEnv):
         self.size = int(params["size"])

@@ -455,6 +455,94 @@ def test_gemm_bf16_17_to_64_tokens(lib, m, n, k, epi):
         assert _rel(out16, want) < 1e-2
 
 
+def _prepared(x, gain):
+    """What epilogue 3 leaves for the norm after it: bf16(x * gain) and the sums of x^2 over
+    every 16 columns, computed the plain way."""
+    t, e = x.shape
+    padded = torch.zeros(t, (e + 15) // 16 * 16, dtype=torch.float64)
+    padded[:, :e] = x.double() ** 2
+    return (x * gain).bfloat16(), padded.view(t, -1, 16).sum(dim=2).float()
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 4096, 4096), (16, 100, 136), (5, 6144, 1024), (8, 8208, 512),
+                                   (3, 9000, 4096), (7, 16400, 8192), (16, 20000, 200), (2, 12288, 1536),
+                                   (4, 520, 14336), (9, 264, 8200)])
+def test_gemm_bf16_few_tokens_folds_sum_and_norm(lib, m, n, k):
+    """The decode products with their neighbours folded in.  As tokens: rows that a product left
+    for a norm (bf16(x * gain) and the sums of x^2 in parts of 16 columns), all of them or chosen
+    ones; the result is that of the normalised rows.  As epilogues: the product added to a
+    float32 matrix, and that with the rows for the next norm left behind.  Sizes cover the
+    streaming kernel with and without bounds checks (K a multiple of 128 or not), 1, 2 and 4 row
+    tiles per wave, a last tile of fewer than 16 columns, counts of sums that are no multiple of
+    4 (K = 136, 200, 8200), more sums than the wide loads take (K = 14336), and the kernel that
+    keeps the tokens in registers (more than 8192 rows of W, K a multiple of 512 up to 4096).
+    The matrix cores see bf16(x * gain), which the first reference repeats; the second is the
+    norm as its own kernel computes it, rounded after the root."""
+    from rbitnet_amd.parts.linear import pack_gate_up
+    assert lib.gemm_bf16_few_ok(m, n, k)
+    g = torch.Generator().manual_seed(m * 11 + n + k)
+    eps = 1e-3
+    pool = torch.randn(m + 5, k, generator=g) * 0.05          # small, so that eps matters
+    gain = 1 + 0.2 * torch.randn(k, generator=g)
+    w = (torch.randn(n, k, generator=g) * 0.5).bfloat16()
+    gained, squares = _prepared(pool, gain)
+    for rows in (None, torch.randperm(m + 5, generator=g)[:m].to(torch.int32)):
+        sel = slice(0, m) if rows is None else rows.long()
+        a = gained[:m].contiguous() if rows is None else gained
+        sq = squares[:m].contiguous() if rows is None else squares
+        picked = pool[sel]
+        scale = 1.0 / torch.sqrt((picked.double() ** 2).mean(dim=1, keepdim=True) + eps)
+        want = (gained[sel].double() @ w.double().T) * scale
+        loose = (picked.double() * gain.double() * scale).float().bfloat16().double() @ w.double().T
+        out = torch.full((m, n), float("nan"), device=DEV, dtype=torch.float32)
+        lib.gemm_bf16_few(a.to(DEV), w.to(DEV), out, 0, squares=sq.to(DEV), eps=eps,
+                          rows=None if rows is None else rows.to(DEV))
+        assert _rel(out, want) < 2e-5, (m, n, k, rows is None)
+        assert _rel(out, loose) < 1e-2
+    # bfloat16 tokens: plain, added to the output, and with the rows for the next norm
+    a = torch.randn(m, k, generator=g).bfloat16()
+    product = a.double() @ w.double().T
+    plain = torch.full((m, n), float("nan"), device=DEV, dtype=torch.float32)
+    lib.gemm_bf16_few(a.to(DEV), w.to(DEV), plain, 0)
+    same = torch.full((m, n), float("nan"), device=DEV, dtype=torch.float32)
+    lib.gemm_bf16(a.to(DEV), w.to(DEV), same, 0)
+    assert torch.equal(plain, same)
+    base = torch.randn(m, n, generator=g)
+    acc = base.to(DEV)
+    lib.gemm_bf16_few(a.to(DEV), w.to(DEV), acc, 2)
+    assert _rel(acc, base.double() + product) < 2e-5
+    next_gain = 1 + 0.2 * torch.randn(n, generator=g)
+    acc3 = base.to(DEV)
+    left = torch.full((m, n), float("nan"), device=DEV, dtype=torch.bfloat16)
+    left_sq = torch.full((m, (n + 15) // 16), float("nan"), device=DEV)
+    lib.gemm_bf16_few(a.to(DEV), w.to(DEV), acc3, 3, gain=next_gain.to(DEV), gained=left, squares_out=left_sq)
+    assert torch.equal(acc3, acc)
+    want_left, want_sq = _prepared(acc3.cpu(), next_gain)
+    assert torch.equal(left.cpu(), want_left)
+    assert _rel(left_sq, want_sq) < 1e-6
+    # prepared rows into the gated epilogue
+    if n % 32 == 0:
+        ff = n // 2
+        wg, wu = w[:ff], w[ff:]
+        scale = 1.0 / torch.sqrt((pool[:m].double() ** 2).mean(dim=1, keepdim=True) + eps)
+        gate = (gained[:m].double() @ wg.double().T) * scale
+        want = gate / (1 + torch.exp(-gate)) * ((gained[:m].double() @ wu.double().T) * scale)
+        out = torch.full((m, ff), float("nan"), device=DEV, dtype=torch.bfloat16)
+        lib.gemm_bf16_few(gained[:m].contiguous().to(DEV), pack_gate_up(wg, wu, True).to(DEV), out, 1,
+                          squares=squares[:m].contiguous().to(DEV), eps=eps)
+        assert _rel(out, want) < 1e-2
+
+
+def test_gemm_bf16_few_refuses_other_sizes(lib):
+    from rbitnet_amd.errors import KernelError
+    assert not lib.gemm_bf16_few_ok(17, 64, 64)
+    assert not lib.gemm_bf16_few_ok(4, 64, 60)
+    a = torch.zeros(17, 64, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(64, 64, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(KernelError, match="not for it"):
+        lib.gemm_bf16_few(a, w, torch.zeros(17, 64, device=DEV), 0)
+
+
 def test_attention_long_context(lib):
     """Thousands of keys over many pages: decode with several split counts and a prompt step
     on top of a long past (chunked prefill), against the plain computation."""
