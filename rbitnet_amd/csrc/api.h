@@ -22,8 +22,10 @@ int rb_embed_gather(const void* table, int table_dtype, const int32_t* ids, floa
 //   src = rows ? rows[r] : r
 //   v = x[src] + (delta ? delta[src] : 0);  if (delta && !rows) x[src] = v
 //   out[r] = v * gain * rsqrt(mean(v^2) + eps)
-int rb_add_rmsnorm(float* x, const float* delta, const float* gain, float eps, const int32_t* rows, int n_rows,
-                   int width, void* out, int out_dtype, void* stream);
+// delta may be n_terms terms, each laid out like x and term_stride floats after the one before:
+// they are added up first, in their order (rb_gemm_bf16_terms leaves such terms).
+int rb_add_rmsnorm(float* x, const float* delta, int n_terms, long long term_stride, const float* gain, float eps,
+                   const int32_t* rows, int n_rows, int width, void* out, int out_dtype, void* stream);
 
 // Rotate q and k by the angle table, write q to q_out and k, v into the cache pages.
 //   qkv      float32 [T, (Hq + 2 Hk) D]: q heads, then k heads, then v heads
@@ -54,6 +56,12 @@ int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dty
 long long rb_gemm_workspace_floats(int m, int n, int k, int epilogue);
 int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
                  float* workspace, void* stream);
+
+// The plain product (float32, epilogue 0) as the terms that the K slices of its kernel computed:
+// terms [rb_gemm_bf16_terms_count(m, n, k), M, N], to be added up in their order.  One term is
+// the product itself.  For a caller that adds them to something else anyway.
+int rb_gemm_bf16_terms_count(int m, int n, int k);
+int rb_gemm_bf16_terms(const void* a, const void* w, float* terms, int m, int n, int k, void* stream);
 
 // The same product for 1..16 tokens with what stands before and after it in a decode step folded
 // in, so that no kernel runs between the products.  rb_gemm_bf16_few_ok: whether it takes these

@@ -47,10 +47,12 @@ extern "C" int rb_embed_gather(const void* table, int table_dtype, const int32_t
 // ---------------------------------------------------------------- add + rmsnorm
 // Reference: s = sum(x^2)/n; scale = 1/sqrt(s + eps); y = x * w * scale
 // (llama/model.rs:93-100); residual adds are plain sums (:292-294, :304-306).
+// delta may be several terms, term_stride floats apart (the partial sums that the K slices of a
+// product left): they are added up first, in their order, and the total is added to x.
 template <typename TO>
-__global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ delta,
-                                   const float* __restrict__ gain, float eps, const int32_t* __restrict__ rows,
-                                   int width, TO* __restrict__ out) {
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ delta, int n_terms,
+                                   size_t term_stride, const float* __restrict__ gain, float eps,
+                                   const int32_t* __restrict__ rows, int width, TO* __restrict__ out) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -58,9 +60,14 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restric
   const float* dr = delta ? delta + src * width : nullptr;
   const bool write_back = (delta != nullptr) && (rows == nullptr);
   float ss = 0.f;
+  auto terms = [&](int j) {
+    float d = dr[j];
+    for (int p = 1; p < n_terms; ++p) d += dr[(size_t)p * term_stride + j];
+    return d;
+  };
   for (int j = threadIdx.x; j < width; j += blockDim.x) {
     float v = xr[j];
-    if (dr) v += dr[j];
+    if (dr) v += terms(j);
     if (write_back) xr[j] = v;
     ss += v * v;
   }
@@ -69,7 +76,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restric
   TO* orow = out + (size_t)r * width;
   for (int j = threadIdx.x; j < width; j += blockDim.x) {
     float v = xr[j];
-    if (dr && !write_back) v += dr[j];
+    if (dr && !write_back) v += terms(j);
     Num<TO>::store(orow + j, v * gain[j] * scale);
   }
 }
@@ -77,8 +84,17 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restric
 // The same for widths that are a multiple of 4 and fit the block's registers: every thread
 // loads its share of the row once with 16-byte loads (the gain too, before the sum is
 // known), so the row makes one trip from memory and the loads are all in flight together.
-template <typename TO, int VPT>          // VPT float4 per thread
-__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta,
+// Several terms are read by four times the threads, each with four terms' loads in flight.
+__device__ __forceinline__ void add4(float4& d, const float4& e) {
+  d.x += e.x;
+  d.y += e.y;
+  d.z += e.z;
+  d.w += e.w;
+}
+
+template <typename TO, int VPT, int THREADS>          // VPT float4 per thread
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta,
+                                                              int n_terms, size_t term_stride,
                                                               const float* __restrict__ gain, float eps,
                                                               const int32_t* __restrict__ rows, int width,
                                                               TO* __restrict__ out) {
@@ -94,16 +110,24 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
-    const int c = threadIdx.x + i * 256;
+    const int c = threadIdx.x + i * THREADS;
     if (c < n4) {
       v[i] = xr[c];
       g[i] = gr[c];
       if (dr) {
-        const float4 d = dr[c];
-        v[i].x += d.x;
-        v[i].y += d.y;
-        v[i].z += d.z;
-        v[i].w += d.w;
+        float4 d = dr[c];
+        const float* term = delta + src * width + 4 * c;
+        auto at = [&](int p) { return *reinterpret_cast<const float4*>(term + (size_t)p * term_stride); };
+        int p = 1;
+        for (; p + 3 < n_terms; p += 4) {
+          const float4 e0 = at(p), e1 = at(p + 1), e2 = at(p + 2), e3 = at(p + 3);
+          add4(d, e0);
+          add4(d, e1);
+          add4(d, e2);
+          add4(d, e3);
+        }
+        for (; p < n_terms; ++p) add4(d, at(p));
+        add4(v[i], d);
       }
     } else {
       v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -112,7 +136,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   }
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
-    const int c = threadIdx.x + i * 256;
+    const int c = threadIdx.x + i * THREADS;
     if (write_back && c < n4) xr[c] = v[i];
     ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
   }
@@ -121,7 +145,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   TO* orow = out + (size_t)r * width;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
-    const int c = threadIdx.x + i * 256;
+    const int c = threadIdx.x + i * THREADS;
     if (c < n4) {
       Num<TO>::store(orow + 4 * c + 0, v[i].x * g[i].x * scale);
       Num<TO>::store(orow + 4 * c + 1, v[i].y * g[i].y * scale);
@@ -132,36 +156,47 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
 }
 
 template <typename TO>
-static bool launch_add_rmsnorm_vec(float* x, const float* delta, const float* gain, float eps, const int32_t* rows,
-                                   int n_rows, int width, TO* out, hipStream_t s) {
-  if (width % 4 != 0) return false;
+static bool launch_add_rmsnorm_vec(float* x, const float* delta, int n_terms, size_t term_stride, const float* gain,
+                                   float eps, const int32_t* rows, int n_rows, int width, TO* out, hipStream_t s) {
+  if (width % 4 != 0 || term_stride % 4 != 0) return false;
   const int n4 = width / 4;
+  if (delta && n_terms > 1 && n4 > 256 && n4 <= 2048) {
+    if (n4 <= 1024)
+      add_rmsnorm_vec_kernel<TO, 1, 1024><<<n_rows, 1024, 0, s>>>(x, delta, n_terms, term_stride, gain, eps, rows, width, out);
+    else
+      add_rmsnorm_vec_kernel<TO, 2, 1024><<<n_rows, 1024, 0, s>>>(x, delta, n_terms, term_stride, gain, eps, rows, width, out);
+    return true;
+  }
   if (n4 <= 256)
-    add_rmsnorm_vec_kernel<TO, 1><<<n_rows, 256, 0, s>>>(x, delta, gain, eps, rows, width, out);
+    add_rmsnorm_vec_kernel<TO, 1, 256><<<n_rows, 256, 0, s>>>(x, delta, n_terms, term_stride, gain, eps, rows, width, out);
   else if (n4 <= 512)
-    add_rmsnorm_vec_kernel<TO, 2><<<n_rows, 256, 0, s>>>(x, delta, gain, eps, rows, width, out);
+    add_rmsnorm_vec_kernel<TO, 2, 256><<<n_rows, 256, 0, s>>>(x, delta, n_terms, term_stride, gain, eps, rows, width, out);
   else if (n4 <= 1024)
-    add_rmsnorm_vec_kernel<TO, 4><<<n_rows, 256, 0, s>>>(x, delta, gain, eps, rows, width, out);
+    add_rmsnorm_vec_kernel<TO, 4, 256><<<n_rows, 256, 0, s>>>(x, delta, n_terms, term_stride, gain, eps, rows, width, out);
   else if (n4 <= 2048)
-    add_rmsnorm_vec_kernel<TO, 8><<<n_rows, 256, 0, s>>>(x, delta, gain, eps, rows, width, out);
+    add_rmsnorm_vec_kernel<TO, 8, 256><<<n_rows, 256, 0, s>>>(x, delta, n_terms, term_stride, gain, eps, rows, width, out);
   else
     return false;
   return true;
 }
 
-extern "C" int rb_add_rmsnorm(float* x, const float* delta, const float* gain, float eps, const int32_t* rows,
-                              int n_rows, int width, void* out, int out_dtype, void* stream) {
+extern "C" int rb_add_rmsnorm(float* x, const float* delta, int n_terms, long long term_stride_ll, const float* gain,
+                              float eps, const int32_t* rows, int n_rows, int width, void* out, int out_dtype,
+                              void* stream) {
   RB_REQUIRE(n_rows >= 0 && width > 0, "rb_add_rmsnorm: bad sizes %d x %d", n_rows, width);
+  RB_REQUIRE(!delta || (n_terms >= 1 && term_stride_ll >= 0), "rb_add_rmsnorm: %d terms, %lld apart", n_terms,
+             term_stride_ll);
+  const size_t term_stride = (size_t)term_stride_ll;
   if (n_rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const int threads = width >= 2048 ? 512 : 256;
-  if (out_dtype == RB_F32 && launch_add_rmsnorm_vec<float>(x, delta, gain, eps, rows, n_rows, width, (float*)out, s)) {
+  if (out_dtype == RB_F32 && launch_add_rmsnorm_vec<float>(x, delta, n_terms, term_stride, gain, eps, rows, n_rows, width, (float*)out, s)) {
   } else if (out_dtype == RB_BF16 &&
-             launch_add_rmsnorm_vec<bf16_t>(x, delta, gain, eps, rows, n_rows, width, (bf16_t*)out, s)) {
+             launch_add_rmsnorm_vec<bf16_t>(x, delta, n_terms, term_stride, gain, eps, rows, n_rows, width, (bf16_t*)out, s)) {
   } else if (out_dtype == RB_F32)
-    add_rmsnorm_kernel<float><<<n_rows, threads, 0, s>>>(x, delta, gain, eps, rows, width, (float*)out);
+    add_rmsnorm_kernel<float><<<n_rows, threads, 0, s>>>(x, delta, n_terms, term_stride, gain, eps, rows, width, (float*)out);
   else if (out_dtype == RB_BF16)
-    add_rmsnorm_kernel<bf16_t><<<n_rows, threads, 0, s>>>(x, delta, gain, eps, rows, width, (bf16_t*)out);
+    add_rmsnorm_kernel<bf16_t><<<n_rows, threads, 0, s>>>(x, delta, n_terms, term_stride, gain, eps, rows, width, (bf16_t*)out);
   else
     RB_REQUIRE(false, "rb_add_rmsnorm: unknown dtype %d", out_dtype);
   RB_LAUNCH_CHECK();

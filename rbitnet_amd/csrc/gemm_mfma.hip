@@ -56,6 +56,23 @@ extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out
   return 0;
 }
 
+// The product as the terms its K slices computed, [terms, M, N] float32, for a caller that adds
+// them up with something else (rb_add_rmsnorm does).  One term: the product itself.
+extern "C" int rb_gemm_bf16_terms_count(int m, int n, int k) {
+  const int p = (m > 0 && n > 0 && k > 0 && k % 8 == 0) ? tiled_parts(m, n, k, 0) : 0;
+  return p > 1 ? p : 1;
+}
+
+extern "C" int rb_gemm_bf16_terms(const void* a, const void* w, float* terms, int m, int n, int k, void* stream) {
+  const int p = rb_gemm_bf16_terms_count(m, n, k);
+  if (p == 1) return rb_gemm_bf16(a, w, terms, RB_F32, 0, m, n, k, nullptr, stream);
+  const int rc = gemm_tiled_launch((const bf16_t*)a, (const bf16_t*)w, nullptr, terms, RB_F32, 0, m, n, k,
+                                   (hipStream_t)stream);
+  if (rc) return rc;
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" int rb_gemm_bf16_few_ok(int m, int n, int k) {
   return m >= 1 && m <= 16 && n > 0 && k > 0 && k % 8 == 0 && tiled_parts(m, n, k, 0) == 0;
 }

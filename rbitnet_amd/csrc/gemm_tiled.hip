@@ -410,7 +410,7 @@ static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int 
   const dim3 grid((unsigned)((tiles + 7) / 8 * 8), (unsigned)parts);
   kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, parts > 1 ? slabs : nullptr, m, n, k, m_tiles,
                                                       n_tiles, k / BK / parts);
-  if (parts > 1) {
+  if (parts > 1 && c != nullptr) {      // without c the caller adds the slabs up itself
     const size_t count = (size_t)m * n;
     gemm_sum_slabs_kernel<TO><<<(unsigned)((count + 255) / 256), 256, 0, s>>>(slabs, (TO*)c, parts, count);
   }

@@ -60,13 +60,15 @@ class Kernels:
         L.rb_last_error.restype = ctypes.c_char_p
         sig = {
             "rb_embed_gather": [_P, _I, _P, _P, _I, _I, _P],
-            "rb_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _I, _P, _I, _P],
+            "rb_add_rmsnorm": [_P, _P, _I, ctypes.c_longlong, _P, _F, _P, _I, _I, _P, _I, _P],
             "rb_rope_kv_write": [_P, _P, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
             "rb_swiglu": [_P, _P, _I, _I, _I, _P],
             "rb_gemm_generic": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
             "rb_gemm_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P],
             "rb_gemm_bf16_few": [_P, _P, _F, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _P],
             "rb_gemm_bf16_few_ok": [_I, _I, _I],
+            "rb_gemm_bf16_terms_count": [_I, _I, _I],
+            "rb_gemm_bf16_terms": [_P, _P, _P, _I, _I, _I, _P],
             "rb_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_prefill_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_decode_bf16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
@@ -112,16 +114,22 @@ class Kernels:
         _check(x, "x", torch.float32)
         if x.shape[1] != width:
             raise KernelError("norm width mismatch")
+        n_terms, term_stride = 1, 0
         if delta is not None:
-            _check(delta, "delta", torch.float32, x.shape)
+            if delta.dim() == 3:            # several terms, to be added up first
+                n_terms, term_stride = delta.shape[0], x.numel()
+                _check(delta, "delta", torch.float32, (n_terms,) + tuple(x.shape))
+            else:
+                _check(delta, "delta", torch.float32, x.shape)
         _check(gain, "gain", torch.float32, (width,))
         if rows is not None:
             _check(rows, "rows", torch.int32, (n_rows,))
         elif x.shape[0] != n_rows:
             raise KernelError("norm row count mismatch")
         _check(out, "out")
-        self._ok(self._lib.rb_add_rmsnorm(_ptr(x), _ptr(delta), _ptr(gain), float(eps), _ptr(rows), n_rows, width,
-                                          _ptr(out), dtype_code(out.dtype), self._stream()))
+        self._ok(self._lib.rb_add_rmsnorm(_ptr(x), _ptr(delta), n_terms, term_stride, _ptr(gain), float(eps),
+                                          _ptr(rows), n_rows, width, _ptr(out), dtype_code(out.dtype),
+                                          self._stream()))
 
     def rope_kv_write(self, qkv, cos, sin, style, q_out, k_pages, v_pages, tok_pos, tok_seq, block_table,
                       n_heads, n_kv, head_dim) -> None:
@@ -172,6 +180,21 @@ class Kernels:
         workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need else None
         self._ok(self._lib.rb_gemm_bf16(_ptr(a), _ptr(w), _ptr(c), dtype_code(c.dtype), int(epilogue), m, n, k,
                                         _ptr(workspace), self._stream()))
+
+    def gemm_bf16_terms_count(self, m: int, n: int, k: int) -> int:
+        return int(self._lib.rb_gemm_bf16_terms_count(int(m), int(n), int(k)))
+
+    def gemm_bf16_terms(self, a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        """a w^T as float32 terms [P, M, N] to be added up in their order: what the K slices of
+        the kernel for these sizes computed (P = 1: the product itself)."""
+        m, k = a.shape
+        n = w.shape[0]
+        _check(a, "a", torch.bfloat16)
+        _check(w, "w", torch.bfloat16, (n, k))
+        terms = torch.empty((int(self._lib.rb_gemm_bf16_terms_count(m, n, k)), m, n), dtype=torch.float32,
+                            device=a.device)
+        self._ok(self._lib.rb_gemm_bf16_terms(_ptr(a), _ptr(w), _ptr(terms), m, n, k, self._stream()))
+        return terms
 
     def gemm_bf16_few_ok(self, m: int, n: int, k: int) -> bool:
         """Whether gemm_bf16_few takes these sizes (1..16 tokens)."""

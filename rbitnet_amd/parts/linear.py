@@ -59,9 +59,15 @@ def linear(lib, x, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
 
 def linear_to_stream(lib, x: torch.Tensor, w: torch.Tensor, stream: Optional[torch.Tensor], next_norm=None):
     """x W^T as a float32 term of the residual stream [M, N].  Without a stream, or where the
-    product cannot add to it itself, the term comes back.  Otherwise it is added, and what comes
-    back is None, or, if the norm that follows folds into products, the `GainedRows` for it."""
+    product cannot add to it itself, the term comes back; as the [P, M, N] partial sums of the
+    kernel's K slices where there are such and the norm that follows `adds_terms`.  Otherwise
+    the product is added, and what comes back is None, or, if the norm that follows folds into
+    products, the `GainedRows` for it."""
     if stream is None or x.shape[0] == 0 or not _few(lib, x, w):
+        m, k = x.shape
+        if (next_norm is not None and getattr(next_norm, "adds_terms", False) and uses_matrix_cores(x.dtype, k)
+                and lib.gemm_bf16_terms_count(m, w.shape[0], k) > 1):
+            return lib.gemm_bf16_terms(x, w)        # [P, M, N]: the norm adds them up with the stream
         return linear(lib, x, w, torch.float32)
     if next_norm is None or not getattr(next_norm, "folds_into_products", False):
         lib.gemm_bf16_few(x, w, stream, 2)

@@ -8,7 +8,8 @@ and the normalised rows come back in the compute dtype.
 
 Interface of a norm: forward(x, delta=None, rows=None) -> h
   x      float32 [T, E], the residual stream; updated in place when delta is given
-  delta  float32 [T, E] or None
+  delta  float32 [T, E] or None; a norm that says `adds_terms` also takes [P, T, E], P terms
+         to be added up in their order
   rows   int32 [R] or None: normalise only these rows (x is then left as it is)
 
 A norm that says `folds_into_products` (with weight, eps and size as here) lets the product
@@ -58,6 +59,7 @@ class GainedRows:
 class RMSNorm(Part):
     graph_safe = True
     folds_into_products = True
+    adds_terms = True
 
     def __init__(self, params: Dict, env: BuildEnv):
         self.size = int(params["size"])

@@ -533,6 +533,42 @@ def test_gemm_bf16_few_tokens_folds_sum_and_norm(lib, m, n, k):
         assert _rel(out, want) < 1e-2
 
 
+@pytest.mark.parametrize("m,n,k", [(40, 4096, 4096), (64, 512, 14336), (300, 1000, 8192), (20, 96, 64), (8, 64, 256)])
+def test_gemm_terms_and_the_norm_that_adds_them(lib, m, n, k):
+    """A product left as the partial sums of its K slices, and the norm that adds them to the
+    stream: the same sums, bit for bit, as the product summed by its own kernel and then
+    added (the terms are added up in the same order).  Sizes with several terms (few tiles, a
+    long K) and with one."""
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16().to(DEV)
+    whole = torch.empty(m, n, device=DEV)
+    lib.gemm_bf16(a, w, whole, 0)
+    terms = lib.gemm_bf16_terms(a, w)
+    assert terms.shape[0] == lib.gemm_bf16_terms_count(m, n, k) and terms.shape[1:] == (m, n)
+    if (m, n, k) in ((40, 4096, 4096), (64, 512, 14336), (300, 1000, 8192)):
+        assert terms.shape[0] > 1
+    total = torch.zeros(m, n, device=DEV)
+    for p in range(terms.shape[0]):
+        total += terms[p]
+    assert torch.equal(total, whole)
+    gain = (1 + 0.1 * torch.randn(n, generator=g)).to(DEV)
+    x0 = torch.randn(m, n, generator=g).to(DEV)
+    for rows in (None, torch.tensor([m - 1, 0, 3], dtype=torch.int32, device=DEV)):
+        r = m if rows is None else 3
+        xa, xb = x0.clone(), x0.clone()
+        ha = torch.empty(r, n, device=DEV, dtype=torch.bfloat16)
+        hb = torch.empty(r, n, device=DEV, dtype=torch.bfloat16)
+        lib.add_rmsnorm(xa, whole, gain, 1e-5, rows, ha)
+        lib.add_rmsnorm(xb, terms, gain, 1e-5, rows, hb)
+        # the stream bit for bit; the rows may differ by a rounding, since the squares of a row
+        # are summed by more threads when there are terms to read
+        assert torch.equal(xa, xb)
+        assert float((ha.float() - hb.float()).abs().max()) <= 2 ** -7 * float(ha.float().abs().max())
+        if rows is None:
+            assert torch.equal(xa, x0 + whole)
+
+
 def test_gemm_bf16_few_refuses_other_sizes(lib):
     from rbitnet_amd.errors import KernelError
     assert not lib.gemm_bf16_few_ok(17, 64, 64)
