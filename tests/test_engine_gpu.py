@@ -88,3 +88,39 @@ def test_unequal_batches_with_slot_reuse(name, dtype):
         for i, r in enumerate(reqs):
             err = max_err(torch.cat(got[i]), plain_logits(name, tuple(r)))
             assert err < TOL[dtype], f"{name} {dtype} round {round_} request {i}: {err}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_batch_that_shrinks_from_20_sequences_to_8(name, dtype):
+    """Steps of more than 16 tokens and of at most 16 run different kernels (with few tokens the
+    products do the residual sums and the norms themselves).  20 sequences decode together,
+    12 of them end after two tokens and the other 8 go on: every sequence's logits match the
+    plain implementation on both sides of the change."""
+    n = 20
+    reqs = [tokens_for(name, 4 + i + (2 if i % 5 < 3 else 6), 40 + i) for i in range(n)]
+    prompt_len = [4 + i for i in range(n)]
+    eng = _engine(name, dtype, max_batch=n, max_tokens=64 * n)
+    slots = [eng.alloc_slot() for _ in reqs]
+    got = [[] for _ in reqs]
+    logits = eng.step([(s, r[:p]) for s, r, p in zip(slots, reqs, prompt_len)], "last")
+    for i in range(n):
+        got[i].append(logits[i:i + 1])
+    done = list(prompt_len)
+    live = list(range(n))
+    sizes = []
+    while live:
+        sizes.append(len(live))
+        logits = eng.step([(slots[i], [reqs[i][done[i]]]) for i in live], "last")
+        for j, i in enumerate(live):
+            got[i].append(logits[j:j + 1])
+            done[i] += 1
+        for i in [i for i in live if done[i] >= len(reqs[i])]:
+            eng.free_slot(slots[i])
+        live = [i for i in live if done[i] < len(reqs[i])]
+    assert sizes == [20, 20, 8, 8, 8, 8]
+    eng.cache.check()
+    for i, r in enumerate(reqs):
+        want = plain_logits(name, tuple(r))[prompt_len[i] - 1:]
+        err = max_err(torch.cat(got[i]), want)
+        assert err < TOL[dtype], f"{name} {dtype} request {i}: {err}"
