@@ -129,6 +129,7 @@ void rb_tune_use_resident(int on);                              // 0: never the 
 void rb_tune_use_stream(int on);                                // 0: the skinny product up to 64 tokens
 void rb_tune_tiles(int cfg, int parts);                         // tiled product: tile configuration and K slices
 void rb_tune_prefill_waves(int waves);                          // prefill attention: 4 or 8
+void rb_tune_prefill_paired(int on);                           // prefill attention: 0 = late blocks first only, no pairing of heavy and light workgroups
 void rb_tune_decode_mfma(int mode);                             // decode attention: 1 matrix cores, 2 vector units
 void rb_tune_decode_waves(int waves);                           // matrix-core decode attention: 4 or 8
 

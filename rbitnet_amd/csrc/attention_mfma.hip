@@ -24,11 +24,11 @@
 
 // =============================================================================== prefill
 template <int D, int NW>
-__global__ __launch_bounds__(64 * NW) void attn_prefill_kernel(
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     bf16_t* __restrict__ out, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ past_len,
     const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, float scale_log2, int window,
-    int gw) {
+    int gw, int paired) {
   constexpr int KLD = D + 8;          // K tile row: D + 8 elements, rows 16 bytes apart in bank space
   constexpr int VLD = RB_PAGE + 8;    // V^T tile row: 64 keys + 8
   constexpr int DC = D / 8;           // 16-byte chunks per row
@@ -42,15 +42,26 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_kernel(
   const int b = blockIdx.z;
   const int group = n_heads / n_kv;
   const int groups_per_kv = group / gw;
-  const int kvh = blockIdx.y / groups_per_kv;
-  const int head = kvh * group + (blockIdx.y % groups_per_kv) * gw + (wave % gw);
+  // Which block of queries and which heads.  The blocks of late queries have the most keys:
+  // they are started first (block index 0 is the last block), and the short ones fill the
+  // compute units that finish early.  `paired`: the workgroups of a sequence, two of which fit
+  // a compute unit, are all resident at once (at most 512 of them); then the first 256 are the
+  // heaviest in falling order and the rest the lightest in rising order, so that the two that
+  // share a compute unit have about the same work together everywhere.
+  int bx = blockIdx.x, by = blockIdx.y;
+  if (paired) {
+    const int n = gridDim.x * gridDim.y, at = blockIdx.x + gridDim.x * blockIdx.y;
+    const int rank = at < 256 ? at : n - 1 - (at - 256);
+    by = rank % gridDim.y;
+    bx = rank / gridDim.y;
+  }
+  const int kvh = by / groups_per_kv;
+  const int head = kvh * group + (by % groups_per_kv) * gw + (wave % gw);
   const int q_per_wg = 32 * (NW / gw);
   const int seq_start = cu_seqlens[b];
   const int q_len = cu_seqlens[b + 1] - seq_start;
   const int past = past_len[b];
-  // the blocks of late queries have the most keys: they are started first, and the short ones
-  // fill the compute units that finish early
-  const int wg_q0 = (gridDim.x - 1 - blockIdx.x) * q_per_wg;
+  const int wg_q0 = (gridDim.x - 1 - bx) * q_per_wg;
   if (wg_q0 >= q_len) return;
   const int q0 = wg_q0 + (wave / gw) * 32;
   const bool wave_on = q0 < q_len;
@@ -254,8 +265,9 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_kernel(
     }
 }
 
-static int g_prefill_waves = 0;
+static int g_prefill_waves = 0, g_prefill_paired = 1;
 extern "C" void rb_tune_prefill_waves(int nw) { g_prefill_waves = nw; }      // experiments only; 0 = built-in
+extern "C" void rb_tune_prefill_paired(int on) { g_prefill_paired = on; }    // experiments only
 
 extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, const void* v_pages, void* out,
                                          const int32_t* cu_seqlens, const int32_t* past_len,
@@ -270,12 +282,17 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
   RB_REQUIRE(window >= 0, "rb_attention_prefill_bf16: negative window");
   const int group = n_heads / n_kv_heads;
   const int gw = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
-  // 8 waves (two per SIMD, which cover each other's softmax arithmetic) when the longest
-  // sequence gives them all queries; 4 for short steps
-  int nw = max_q_len > 32 * (4 / gw) ? 8 : 4;
+  // Workgroups of 4 waves, two of which share a compute unit (their waves cover each other's
+  // softmax arithmetic), or of 8 waves with twice the queries, which stage every tile of keys
+  // and values for twice the work.  Measured with 32 heads on 8 kv heads, head size 128: the
+  // small ones are faster up to about 12k tokens (2,048: 74 us against 86, where 256 large
+  // workgroups run in one round and the last block of queries sets the time; 8,192: 820
+  // against 900), the large ones beyond (32,768: 9.7 ms against 10.3).
+  int nw = max_q_len <= 8192 ? 4 : 8;
   if (g_prefill_waves) nw = g_prefill_waves;
   const int q_per_wg = 32 * (nw / gw);
   dim3 grid((max_q_len + q_per_wg - 1) / q_per_wg, n_kv_heads * (group / gw), n_seqs);
+  const int paired = (nw == 4 && g_prefill_paired && grid.x * grid.y > 256 && grid.x * grid.y <= 512) ? 1 : 0;
   RB_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "rb_attention_prefill_bf16: batch or head count too large");
   hipStream_t s = (hipStream_t)stream;
   const float sl2 = scale * LOG2E;
@@ -283,7 +300,7 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
   attn_prefill_kernel<DV, NWV><<<grid, 64 * NWV, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages,              \
                                                          (const bf16_t*)v_pages, (bf16_t*)out, cu_seqlens,      \
                                                          past_len, block_table, bt_stride, n_heads, n_kv_heads, \
-                                                         sl2, window, gw)
+                                                         sl2, window, gw, paired)
   if (head_dim == 128) {
     if (nw == 8) RB_PF(128, 8);
     else RB_PF(128, 4);

@@ -286,6 +286,56 @@ def test_attention_prefill_bf16(lib, n_heads, n_kv, d, window):
     assert _rel(out, want) < 1.5e-2
 
 
+@pytest.mark.parametrize("waves", [0, 8])
+@pytest.mark.parametrize("n_heads,n_kv,d,t,window", [(24, 24, 64, 1536, 0), (32, 8, 128, 1100, 0), (8, 2, 128, 2500, 300),
+                                                    (4, 4, 64, 700, 0)])
+def test_attention_prefill_of_a_long_prompt(lib, waves, n_heads, n_kv, d, t, window):
+    """One prompt of a thousand tokens and more, where the order in which the workgroups take
+    the blocks of queries matters: between 257 and 512 workgroups a sequence (288, 280 and 316
+    in the first three cases) the heaviest and the lightest blocks are paired; the last case
+    has fewer.  waves = 8: the kernel with twice the queries per workgroup, which the
+    library takes only beyond 8,192 tokens.  Every row of the output is compared."""
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(t + n_heads)
+    n_pages = (t + 63) // 64
+    q = (torch.randn(t, n_heads, d, generator=g) * 1.5).to(dtype)
+    k = torch.randn(t, n_kv, d, generator=g).to(dtype)
+    v = torch.randn(t, n_kv, d, generator=g).to(dtype)
+    order = torch.randperm(n_pages, generator=g).to(torch.int32)          # the pages lie anywhere
+    kp = torch.full((n_pages, n_kv, 64, d), float("nan"), dtype=dtype)
+    vp = torch.full((n_pages, n_kv, 64, d), float("nan"), dtype=dtype)
+    for pg in range(n_pages):
+        rows = slice(64 * pg, min(64 * pg + 64, t))
+        kp[int(order[pg]), :, :rows.stop - rows.start] = k[rows].transpose(0, 1)
+        vp[int(order[pg]), :, :rows.stop - rows.start] = v[rows].transpose(0, 1)
+    out = torch.full((t, n_heads * d), float("nan"), dtype=dtype, device=DEV)
+    cu = torch.tensor([0, t], dtype=torch.int32, device=DEV)
+    scale = 1 / math.sqrt(d)
+    lib._lib.rb_tune_prefill_waves(waves)
+    try:
+        lib.attention_prefill_bf16(q.to(DEV), kp.to(DEV), vp.to(DEV), out, cu,
+                                   torch.zeros(1, dtype=torch.int32, device=DEV), order.view(1, -1).to(DEV), 1, t,
+                                   n_heads, n_kv, d, scale, window)
+    finally:
+        lib._lib.rb_tune_prefill_waves(0)
+    # plain attention in float64 (on the GPU, for its speed)
+    qd, kd, vd = q.to(DEV).double(), k.to(DEV).double(), v.to(DEV).double()
+    pos = torch.arange(t, device=DEV)
+    seen = pos[None, :] <= pos[:, None]
+    if window:
+        seen &= pos[None, :] > pos[:, None] - window
+    want = torch.empty(t, n_heads, d, dtype=torch.float64, device=DEV)
+    for h in range(n_heads):
+        kvh = h // (n_heads // n_kv)
+        scores = (qd[:, h] @ kd[:, kvh].T) * scale
+        scores = scores.masked_fill(~seen, float("-inf"))
+        want[:, h] = torch.softmax(scores, dim=1) @ vd[:, kvh]
+    got = out.double().view(t, n_heads, d)
+    assert bool(torch.isfinite(got).all())
+    err = (got - want).abs().amax(dim=(1, 2)) / want.abs().amax()
+    assert float(err.max()) < 1.5e-2, int(err.argmax())
+
+
 @pytest.fixture
 def decode_kernel(lib, request):
     """"auto": the kernel the library picks for the group size; "matrix": the matrix-core
