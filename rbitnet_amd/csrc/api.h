@@ -28,13 +28,14 @@ int rb_add_rmsnorm(float* x, const float* delta, int n_terms, long long term_str
                    const int32_t* rows, int n_rows, int width, void* out, int out_dtype, void* stream);
 
 // Rotate q and k by the angle table, write q to q_out and k, v into the cache pages.
-//   qkv      float32 [T, (Hq + 2 Hk) D]: q heads, then k heads, then v heads
+//   qkv      float32 [T, (Hq + 2 Hk) D]: q heads, then k heads, then v heads; as qkv_terms terms
+//            to be added up in their order, qkv_term_stride floats apart (1 term: qkv itself)
 //   cos, sin float32 [max_pos, D/2], or null for no rotation
 //   style    0: pairs (2i, 2i+1); 1: pairs (i, i + D/2)
 //   k_pages, v_pages [n_pages, Hk, 64, D] of cache_dtype; null when the layer keeps no cache
 //   tok_pos, tok_seq int32 [T]; block_table int32 [B, bt_stride]
-int rb_rope_kv_write(const float* qkv, const float* cos, const float* sin, int style, void* q_out, void* k_pages,
-                     void* v_pages, int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq,
+int rb_rope_kv_write(const float* qkv, int qkv_terms, long long qkv_term_stride, const float* cos, const float* sin,
+                     int style, void* q_out, void* k_pages, void* v_pages, int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq,
                      const int32_t* block_table, int bt_stride, int n_tokens, int n_heads, int n_kv_heads,
                      int head_dim, void* stream);
 
@@ -102,8 +103,9 @@ int rb_attention_decode_bf16(const void* q, const void* k_pages, const void* v_p
 //   decode, fused: rotation of q and the new k, cache write and attention in one kernel (plus the
 //   combination of the splits when there are several).  qkv float32 [B, (Hq + 2 Hk) D] as for
 //   rb_rope_kv_write.
-int rb_attention_decode_fused_bf16(const float* qkv, const float* cos, const float* sin, int style, void* k_pages,
-                                   void* v_pages, void* out, const int32_t* tok_pos, const int32_t* block_table,
+int rb_attention_decode_fused_bf16(const float* qkv, int qkv_terms, long long qkv_term_stride, const float* cos,
+                                   const float* sin, int style, void* k_pages, void* v_pages, void* out,
+                                   const int32_t* tok_pos, const int32_t* block_table,
                                    int bt_stride, int n_seqs, int n_heads, int n_kv_heads, int head_dim, float scale,
                                    int window, int n_splits, float* workspace, void* stream);
 

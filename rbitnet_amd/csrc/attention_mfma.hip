@@ -384,7 +384,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const float* __restrict__ qkv, const bf16_t* __restrict__ q_in, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int style, bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
-    int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws) {
+    int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws, int qkv_terms, size_t qkv_stride) {
   constexpr int DL = D / 64;          // output elements per lane
   constexpr int QC = D / 32;          // 16-byte chunks of a quarter row of K
   constexpr int QP = D / 8;           // bfloat16 pairs of a quarter row
@@ -414,7 +414,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       const int gg = idx / HALF, i = idx - gg * HALF;
       const int i0 = style == 0 ? 2 * i : i, i1 = style == 0 ? 2 * i + 1 : i + HALF;
       const float* h = gg < G ? src + (size_t)(kvh * G + gg) * D : src + (size_t)(n_heads + kvh) * D;
-      const float x0 = h[i0], x1 = h[i1];
+      const float x0 = sum_terms(h + i0, qkv_terms, qkv_stride), x1 = sum_terms(h + i1, qkv_terms, qkv_stride);
       float y0 = x0, y1 = x1;
       if (cr) {
         const float c = cr[i], sn = sr[i];
@@ -425,7 +425,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       dst[i0] = f32_to_bf16_bits(y0);
       dst[i1] = f32_to_bf16_bits(y1);
     }
-    for (int d = tid; d < D; d += 256) vnew_h[d] = f32_to_bf16_bits(src[(size_t)(n_heads + n_kv + kvh) * D + d]);
+    for (int d = tid; d < D; d += 256)
+      vnew_h[d] = f32_to_bf16_bits(sum_terms(src + (size_t)(n_heads + n_kv + kvh) * D + d, qkv_terms, qkv_stride));
     __syncthreads();
 #pragma unroll
     for (int gg = 0; gg < G; ++gg)
@@ -634,7 +635,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
     const float* __restrict__ qkv, const bf16_t* __restrict__ q_in, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int style, bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
-    int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws) {
+    int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws, int qkv_terms, size_t qkv_stride) {
   constexpr int KS = D / 32;          // depth steps of the score product
   constexpr int DT = D / 16;          // d tiles of the output product
   constexpr int HALF = D / 2;
@@ -678,7 +679,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
         continue;
       }
       const float* h = gg < 16 ? src + (size_t)(kvh * G + gg) * D : src + (size_t)(n_heads + kvh) * D;
-      const float x0 = h[i0], x1 = h[i1];
+      const float x0 = sum_terms(h + i0, qkv_terms, qkv_stride), x1 = sum_terms(h + i1, qkv_terms, qkv_stride);
       float y0 = x0, y1 = x1;
       if (cr) {
         const float c = cr[i], sn = sr[i];
@@ -688,7 +689,8 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
       dst[i0] = f32_to_bf16_bits(y0);
       dst[i1] = f32_to_bf16_bits(y1);
     }
-    for (int d = tid; d < D; d += NT) vnew_h[d] = f32_to_bf16_bits(src[(size_t)(n_heads + n_kv + kvh) * D + d]);
+    for (int d = tid; d < D; d += NT)
+      vnew_h[d] = f32_to_bf16_bits(sum_terms(src + (size_t)(n_heads + n_kv + kvh) * D + d, qkv_terms, qkv_stride));
   } else {
     for (int idx = tid; idx < 16 * D; idx += NT) {
       const int gg = idx / D, d = idx - gg * D;
@@ -899,6 +901,8 @@ struct DecodeArgs {
   float sl2;
   int window, n_splits;
   float* ws;
+  int qkv_terms;          // fused: qkv as so many terms to be added up, qkv_stride floats apart
+  size_t qkv_stride;
 };
 
 template <int D, int G, bool FUSED>
@@ -906,7 +910,7 @@ static void launch_decode(const DecodeArgs& a, hipStream_t s) {
   dim3 grid(a.n_splits, a.n_kv, a.n_seqs);
   attn_decode_kernel<D, G, FUSED><<<grid, 256, 0, s>>>(a.qkv, a.q, a.cos_t, a.sin_t, a.style, a.k, a.v, a.out,
                                                        a.tok_pos, a.bt, a.bt_stride, a.n_heads, a.n_kv, a.sl2,
-                                                       a.window, a.n_splits, a.ws);
+                                                       a.window, a.n_splits, a.ws, a.qkv_terms, a.qkv_stride);
   if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits);
 }
 
@@ -923,7 +927,8 @@ static int launch_decode_mfma_nw(const DecodeArgs& a, hipStream_t s) {
   }
   dim3 grid(a.n_splits, a.n_kv, a.n_seqs);
   kern<<<grid, 64 * NW, lds, s>>>(a.qkv, a.q, a.cos_t, a.sin_t, a.style, a.k, a.v, a.out, a.tok_pos, a.bt,
-                                  a.bt_stride, a.n_heads, a.n_kv, a.sl2, a.window, a.n_splits, a.ws);
+                                  a.bt_stride, a.n_heads, a.n_kv, a.sl2, a.window, a.n_splits, a.ws, a.qkv_terms,
+                                  a.qkv_stride);
   if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits);
   return 0;
 }
@@ -991,19 +996,22 @@ extern "C" int rb_attention_decode_bf16(const void* q, const void* k_pages, cons
                                         int window, int n_splits, float* workspace, void* stream) {
   DecodeArgs a = {nullptr, (const bf16_t*)q, nullptr, nullptr, 0, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out,
                   tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, scale * LOG2E, window, n_splits,
-                  workspace};
+                  workspace, 1, 0};
   return dispatch_decode<false>(a, head_dim, (hipStream_t)stream, "rb_attention_decode_bf16");
 }
 
-extern "C" int rb_attention_decode_fused_bf16(const float* qkv, const float* cos, const float* sin, int style,
+extern "C" int rb_attention_decode_fused_bf16(const float* qkv, int qkv_terms, long long qkv_term_stride,
+                                              const float* cos, const float* sin, int style,
                                               void* k_pages, void* v_pages, void* out, const int32_t* tok_pos,
                                               const int32_t* block_table, int bt_stride, int n_seqs, int n_heads,
                                               int n_kv_heads, int head_dim, float scale, int window, int n_splits,
                                               float* workspace, void* stream) {
   RB_REQUIRE((cos == nullptr) == (sin == nullptr), "rb_attention_decode_fused_bf16: cos and sin tables go together");
   RB_REQUIRE(style == 0 || style == 1, "rb_attention_decode_fused_bf16: unknown pairing style %d", style);
+  RB_REQUIRE(qkv_terms >= 1 && qkv_term_stride >= 0, "rb_attention_decode_fused_bf16: %d terms, %lld apart", qkv_terms,
+             qkv_term_stride);
   DecodeArgs a = {qkv, nullptr, cos, sin, style, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out,
                   tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, scale * LOG2E, window, n_splits,
-                  workspace};
+                  workspace, qkv_terms, (size_t)qkv_term_stride};
   return dispatch_decode<true>(a, head_dim, (hipStream_t)stream, "rb_attention_decode_fused_bf16");
 }

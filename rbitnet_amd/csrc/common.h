@@ -76,6 +76,25 @@ struct Num<bf16_t> {
   static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 };
 
+// ---------------------------------------------------------------- terms of a product
+// A product whose K was cut into slices may be left as its slices' sums, `stride` floats
+// apart: p[0] + p[stride] + ... in that order (the order in which the product's own kernel
+// adds them), four loads in flight.
+__device__ __forceinline__ float sum_terms(const float* __restrict__ p, int n_terms, size_t stride) {
+  float v = p[0];
+  int t = 1;
+  for (; t + 3 < n_terms; t += 4) {
+    const float e0 = p[(size_t)t * stride], e1 = p[(size_t)(t + 1) * stride], e2 = p[(size_t)(t + 2) * stride],
+                e3 = p[(size_t)(t + 3) * stride];
+    v += e0;
+    v += e1;
+    v += e2;
+    v += e3;
+  }
+  for (; t < n_terms; ++t) v += p[(size_t)t * stride];
+  return v;
+}
+
 // ---------------------------------------------------------------- reductions
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -208,7 +208,8 @@ extern "C" int rb_add_rmsnorm(float* x, const float* delta, int n_terms, long lo
 //   x0' = x0 cos - x1 sin, x1' = x0 sin + x1 cos (llama/model.rs:122-136), for every q
 // head and k head (:242-252); k is cached rotated, v as it is (:254-257).
 template <typename TC>
-__global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const float* __restrict__ cos_t,
+__global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int n_terms, size_t term_stride,
+                                     const float* __restrict__ cos_t,
                                      const float* __restrict__ sin_t, int style, TC* __restrict__ q_out,
                                      TC* __restrict__ k_pages, TC* __restrict__ v_pages,
                                      const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
@@ -233,8 +234,8 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const float*
     const int i = idx - h * half;
     const int i0 = style == 0 ? 2 * i : i;
     const int i1 = style == 0 ? 2 * i + 1 : i + half;
-    const float x0 = src[h * head_dim + i0];
-    const float x1 = src[h * head_dim + i1];
+    const float x0 = sum_terms(src + h * head_dim + i0, n_terms, term_stride);
+    const float x1 = sum_terms(src + h * head_dim + i1, n_terms, term_stride);
     float y0 = x0, y1 = x1;
     if (cr) {
       const float c = cr[i], s = sr[i];
@@ -256,28 +257,32 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const float*
     for (int idx = threadIdx.x; idx < n_kv * head_dim; idx += blockDim.x) {
       const int h = idx / head_dim;
       const int d = idx - h * head_dim;
-      Num<TC>::store(v_pages + page_base + (size_t)h * RB_PAGE * head_dim + d, vsrc[idx]);
+      Num<TC>::store(v_pages + page_base + (size_t)h * RB_PAGE * head_dim + d,
+                     sum_terms(vsrc + idx, n_terms, term_stride));
     }
   }
 }
 
-extern "C" int rb_rope_kv_write(const float* qkv, const float* cos, const float* sin, int style, void* q_out,
+extern "C" int rb_rope_kv_write(const float* qkv, int qkv_terms, long long qkv_term_stride, const float* cos,
+                                const float* sin, int style, void* q_out,
                                 void* k_pages, void* v_pages, int cache_dtype, const int32_t* tok_pos,
                                 const int32_t* tok_seq, const int32_t* block_table, int bt_stride, int n_tokens,
                                 int n_heads, int n_kv_heads, int head_dim, void* stream) {
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0 && head_dim % 2 == 0,
              "rb_rope_kv_write: bad sizes T=%d Hq=%d Hk=%d D=%d", n_tokens, n_heads, n_kv_heads, head_dim);
+  RB_REQUIRE(qkv_terms >= 1 && qkv_term_stride >= 0, "rb_rope_kv_write: %d terms, %lld apart", qkv_terms,
+             qkv_term_stride);
   RB_REQUIRE((cos == nullptr) == (sin == nullptr), "rb_rope_kv_write: cos and sin tables go together");
   RB_REQUIRE(style == 0 || style == 1, "rb_rope_kv_write: unknown pairing style %d", style);
   RB_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rb_rope_kv_write: k and v pages go together");
   if (n_tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (cache_dtype == RB_F32)
-    rope_kv_write_kernel<float><<<n_tokens, 256, 0, s>>>(qkv, cos, sin, style, (float*)q_out, (float*)k_pages,
+    rope_kv_write_kernel<float><<<n_tokens, 256, 0, s>>>(qkv, qkv_terms, (size_t)qkv_term_stride, cos, sin, style, (float*)q_out, (float*)k_pages,
                                                          (float*)v_pages, tok_pos, tok_seq, block_table,
                                                          bt_stride, n_heads, n_kv_heads, head_dim);
   else if (cache_dtype == RB_BF16)
-    rope_kv_write_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(qkv, cos, sin, style, (bf16_t*)q_out,
+    rope_kv_write_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(qkv, qkv_terms, (size_t)qkv_term_stride, cos, sin, style, (bf16_t*)q_out,
                                                           (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, tok_seq,
                                                           block_table, bt_stride, n_heads, n_kv_heads, head_dim);
   else

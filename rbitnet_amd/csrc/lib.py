@@ -43,6 +43,17 @@ def _check(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
         raise KernelError(f"{name} must have shape {tuple(shape)}, found {tuple(t.shape)}")
 
 
+def _terms(qkv: torch.Tensor, width: int):
+    """qkv [T, width], or [P, T, width]: P terms to be added up in their order.  -> (T, P, stride)"""
+    if qkv.dim() == 3:
+        p, n = qkv.shape[0], qkv.shape[1]
+        _check(qkv, "qkv", torch.float32, (p, n, width))
+        return n, p, n * width
+    n = qkv.shape[0]
+    _check(qkv, "qkv", torch.float32, (n, width))
+    return n, 1, 0
+
+
 class Kernels:
     """The loaded library.  Methods check operand shapes on the host before a launch, so
     that a kernel never sees sizes other than the ones its grid assumes."""
@@ -61,7 +72,7 @@ class Kernels:
         sig = {
             "rb_embed_gather": [_P, _I, _P, _P, _I, _I, _P],
             "rb_add_rmsnorm": [_P, _P, _I, ctypes.c_longlong, _P, _F, _P, _I, _I, _P, _I, _P],
-            "rb_rope_kv_write": [_P, _P, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "rb_rope_kv_write": [_P, _I, ctypes.c_longlong, _P, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
             "rb_swiglu": [_P, _P, _I, _I, _I, _P],
             "rb_gemm_generic": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
             "rb_gemm_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P],
@@ -72,7 +83,7 @@ class Kernels:
             "rb_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_prefill_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_decode_bf16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
-            "rb_attention_decode_fused_bf16": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
+            "rb_attention_decode_fused_bf16": [_P, _I, ctypes.c_longlong, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
                                                _P, _P],
             "rb_sample": [_P, _I, _I, _P, _P, _P, _P, _P],
             "rb_probe_read": [_P, ctypes.c_longlong, _I, _P, _P],
@@ -133,8 +144,7 @@ class Kernels:
 
     def rope_kv_write(self, qkv, cos, sin, style, q_out, k_pages, v_pages, tok_pos, tok_seq, block_table,
                       n_heads, n_kv, head_dim) -> None:
-        n = qkv.shape[0]
-        _check(qkv, "qkv", torch.float32, (n, (n_heads + 2 * n_kv) * head_dim))
+        n, n_terms, term_stride = _terms(qkv, (n_heads + 2 * n_kv) * head_dim)
         _check(q_out, "q_out", None, (n, n_heads, head_dim))
         _check(tok_pos, "tok_pos", torch.int32, (n,))
         _check(tok_seq, "tok_seq", torch.int32, (n,))
@@ -150,8 +160,9 @@ class Kernels:
             if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, head_dim):
                 raise KernelError(f"cache pages have shape {tuple(k_pages.shape)}, expected "
                                   f"[*, {n_kv}, {self.page_size}, {head_dim}]")
-        self._ok(self._lib.rb_rope_kv_write(_ptr(qkv), _ptr(cos), _ptr(sin), int(style), _ptr(q_out), _ptr(k_pages),
-                                            _ptr(v_pages), dtype_code(q_out.dtype), _ptr(tok_pos), _ptr(tok_seq),
+        self._ok(self._lib.rb_rope_kv_write(_ptr(qkv), n_terms, term_stride, _ptr(cos), _ptr(sin), int(style),
+                                            _ptr(q_out), _ptr(k_pages), _ptr(v_pages), dtype_code(q_out.dtype),
+                                            _ptr(tok_pos), _ptr(tok_seq),
                                             _ptr(block_table), block_table.shape[1], n, n_heads, n_kv, head_dim,
                                             self._stream()))
 
@@ -284,8 +295,7 @@ class Kernels:
 
     def attention_decode_fused_bf16(self, qkv, cos, sin, style, k_pages, v_pages, out, tok_pos, block_table,
                                     n_heads, n_kv, head_dim, scale, window, n_splits, workspace) -> None:
-        n = qkv.shape[0]
-        _check(qkv, "qkv", torch.float32, (n, (n_heads + 2 * n_kv) * head_dim))
+        n, n_terms, term_stride = _terms(qkv, (n_heads + 2 * n_kv) * head_dim)
         if cos is not None:
             _check(cos, "cos", torch.float32)
             _check(sin, "sin", torch.float32, cos.shape)
@@ -302,7 +312,8 @@ class Kernels:
         if workspace.numel() < n * n_heads * n_splits * (head_dim + 2):
             raise KernelError("decode attention workspace too small")
         self._ok(self._lib.rb_attention_decode_fused_bf16(
-            _ptr(qkv), _ptr(cos), _ptr(sin), int(style), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tok_pos),
+            _ptr(qkv), n_terms, term_stride, _ptr(cos), _ptr(sin), int(style), _ptr(k_pages), _ptr(v_pages), _ptr(out),
+            _ptr(tok_pos),
             _ptr(block_table), block_table.shape[1], n, n_heads, n_kv, head_dim, float(scale), int(window or 0),
             int(n_splits), _ptr(workspace), self._stream()))
 

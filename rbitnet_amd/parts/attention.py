@@ -32,7 +32,7 @@ import torch
 
 from ..errors import ConfigError, KernelError
 from .base import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register_mixer
-from .linear import linear, linear_to_stream
+from .linear import linear, linear_or_terms, linear_to_stream
 
 DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight"}
 _MATRIX_CORE_HEAD_DIMS = (64, 128)
@@ -95,7 +95,11 @@ class Attention(Part):
         t = h.shape[0]
         hq, hk, d = self.n_heads, self.n_kv, self.head_dim
         owns = self.cache_from is None
-        qkv = linear(lib, h, self.w_qkv, torch.float32)
+        # q, k and v of the step; as the terms of the product where the position part reads such
+        if getattr(self.position, "takes_terms", False):
+            qkv = linear_or_terms(lib, h, self.w_qkv)
+        else:
+            qkv = linear(lib, h, self.w_qkv, torch.float32)
         bt = view.block_table
         attn = torch.empty((t, hq * d), dtype=self.env.dtype, device=h.device)
         window = int(self.window) if self.window is not None else 0

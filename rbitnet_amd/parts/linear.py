@@ -57,6 +57,15 @@ def linear(lib, x, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+def linear_or_terms(lib, x, w: torch.Tensor) -> torch.Tensor:
+    """x W^T in float32 for a reader that adds up terms itself: [M, N], or [P, M, N] where the
+    product's kernel cut K into P slices (their sums are then not added by a kernel of their own)."""
+    if (not isinstance(x, GainedRows) and x.shape[0] > 0 and uses_matrix_cores(x.dtype, x.shape[1])
+            and lib.gemm_bf16_terms_count(x.shape[0], w.shape[0], x.shape[1]) > 1):
+        return lib.gemm_bf16_terms(x, w)
+    return linear(lib, x, w, torch.float32)
+
+
 def linear_to_stream(lib, x: torch.Tensor, w: torch.Tensor, stream: Optional[torch.Tensor], next_norm=None):
     """x W^T as a float32 term of the residual stream [M, N].  Without a stream, or where the
     product cannot add to it itself, the term comes back; as the [P, M, N] partial sums of the

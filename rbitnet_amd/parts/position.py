@@ -5,6 +5,8 @@ Interface: encode_and_store(qkv, q_out, k_pages, v_pages, ctx, block_table,
                             n_heads, n_kv_heads, head_dim)
 Optional:  rotation_tables() -> (cos, sin, style) when the encoding is a per-position,
            per-pair rotation; a mixer may then apply it inside a fused kernel.
+           takes_terms = True: qkv may also be [P, T, W], the sums of the K slices of the
+           product that made it, which encode_and_store adds up in their order as it reads.
 
 "rope": the rotation of the reference (crates/bitnet-core/src/llama/model.rs:122-136):
 inv_i = 1 / theta^(2i/D), angle = pos * inv_i, pairs (x[2i], x[2i+1]) ("interleaved") or
@@ -53,6 +55,7 @@ def rope_inverse_frequencies(head_dim: int, theta: float, scaling: Optional[Dict
 
 class Rope(Part):
     graph_safe = True
+    takes_terms = True      # qkv may come as [P, T, W]: terms that the kernel adds up
 
     def __init__(self, params: Dict, env: BuildEnv):
         self.head_dim = int(params["head_dim"])
@@ -87,6 +90,7 @@ class Rope(Part):
 
 class NoPosition(Part):
     graph_safe = True
+    takes_terms = True
 
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env

@@ -247,6 +247,19 @@ def test_rope_kv_write(lib, style, dtype):
         page = int(bt[b, pos // 64])
         assert _rel(kp[page, :, pos % 64], rot[n_heads:]) < tol
         assert _rel(vp[page, :, pos % 64], heads[n_heads + n_kv:]) < tol
+    # qkv as the terms of a product whose K was cut into slices: added up in their order
+    for n_terms in (2, 7):
+        terms = torch.randn(n_terms, *qkv.shape, generator=g)
+        total = terms[0].clone()
+        for p in range(1, n_terms):
+            total += terms[p]
+        kp1, vp1, qo1 = torch.zeros_like(kp), torch.zeros_like(vp), torch.empty_like(qo)
+        kp2, vp2, qo2 = torch.zeros_like(kp), torch.zeros_like(vp), torch.empty_like(qo)
+        lib.rope_kv_write(total.to(DEV), cos.to(DEV), sin.to(DEV), style, qo1, kp1, vp1, tok_pos.to(DEV),
+                          tok_seq.to(DEV), bt.to(DEV), n_heads, n_kv, d)
+        lib.rope_kv_write(terms.to(DEV), cos.to(DEV), sin.to(DEV), style, qo2, kp2, vp2, tok_pos.to(DEV),
+                          tok_seq.to(DEV), bt.to(DEV), n_heads, n_kv, d)
+        assert torch.equal(qo1, qo2) and torch.equal(kp1, kp2) and torch.equal(vp1, vp2)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -472,6 +485,29 @@ def test_attention_decode_fused_bf16(lib, n_heads, n_kv, d, window, n_splits, st
         for b in range(nb):
             page, off = int(bt[b, past[b] // 64]), past[b] % 64
             assert torch.equal(kp[page, :, off].cpu(), k_new[b]) and torch.equal(vp[page, :, off].cpu(), v_new[b])
+        if call == 0:
+            # qkv as 6 terms that add up (in their order) to the same numbers: the same result, bit for bit
+            parts = torch.randn(5, *qkv.shape, generator=g)
+            rest = qkv.clone()
+            for p in range(5):
+                rest -= parts[p]
+            terms = torch.cat([parts, rest[None]])
+            total = terms[0].clone()
+            for p in range(1, 6):
+                total += terms[p]
+            kp1, vp1 = _fill_pages(k_past, v_past, bt, 64, n_kv, d, dtype)
+            kp2, vp2 = _fill_pages(k_past, v_past, bt, 64, n_kv, d, dtype)
+            kp1, vp1, kp2, vp2 = kp1.to(DEV), vp1.to(DEV), kp2.to(DEV), vp2.to(DEV)
+            out1, out2 = torch.empty_like(out), torch.empty_like(out)
+            lib.attention_decode_fused_bf16(total.to(DEV), cos, sin, style, kp1, vp1, out1, tok_pos.to(DEV),
+                                            bt.to(DEV), n_heads, n_kv, d, scale, window, n_splits, ws)
+            lib.attention_decode_fused_bf16(terms.to(DEV), cos, sin, style, kp2, vp2, out2, tok_pos.to(DEV),
+                                            bt.to(DEV), n_heads, n_kv, d, scale, window, n_splits, ws)
+            assert torch.equal(out1, out2)
+            for b in range(nb):
+                page, off = int(bt[b, past[b] // 64]), past[b] % 64
+                assert torch.equal(kp1[page, :, off], kp2[page, :, off])
+                assert torch.equal(vp1[page, :, off], vp2[page, :, off])
 
 
 @pytest.mark.parametrize("m", [17, 31, 48, 64])
