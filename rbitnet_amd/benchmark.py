@@ -18,7 +18,6 @@ from __future__ import annotations
 
 import argparse
 import json
-import sys
 import time
 
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}

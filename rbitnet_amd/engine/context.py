@@ -7,7 +7,7 @@ past_len[b], past_len[b] + 1, ...
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Dict, List, Sequence, Tuple
 
 import numpy as np
 import torch

@@ -12,14 +12,13 @@ the model's or the cache's limit are errors raised before anything is launched.
 """
 from __future__ import annotations
 
-import os
 from typing import Any, Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
 from ..cache import PAGE_SIZE, Cache, pages_for
 from ..config import load_config
-from ..errors import CacheError, ConfigError, InferenceError, KernelError
+from ..errors import ConfigError, InferenceError
 from ..weights import DEFAULT_SEED, RandomTensors, load_weights
 from .context import StepContext
 from .model import Model

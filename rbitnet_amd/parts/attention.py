@@ -30,7 +30,7 @@ from typing import Dict, Optional
 
 import torch
 
-from ..errors import ConfigError, KernelError
+from ..errors import ConfigError
 from .base import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register_mixer
 from .linear import linear, linear_or_terms, linear_to_stream
 

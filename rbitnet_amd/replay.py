@@ -20,7 +20,6 @@ import os
 import sys
 from typing import Dict, IO, Optional
 
-import numpy as np
 
 from .errors import RbitnetError
 

@@ -13,7 +13,7 @@ import hashlib
 import json
 import os
 from collections.abc import Mapping
-from typing import Any, Dict, Iterator, Optional, Tuple
+from typing import Any, Dict, Iterator, Tuple
 
 import torch
 

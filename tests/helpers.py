@@ -1,7 +1,6 @@
 """Tiny configurations, model folders and oracle logits shared by the tests."""
 from __future__ import annotations
 
-import json
 import os
 import tempfile
 from functools import lru_cache

@@ -5,7 +5,7 @@ import random
 import pytest
 import torch
 
-from rbitnet_amd.cache import PAGE_SIZE, Cache, FreeList, PageTable, pages_for
+from rbitnet_amd.cache import PAGE_SIZE, Cache, FreeList, pages_for
 from rbitnet_amd.errors import CacheError, InferenceError
 from rbitnet_amd.parts.base import CacheRequest
 

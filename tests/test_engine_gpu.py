@@ -3,7 +3,7 @@ the last 32 tokens one by one, and batches of unequal lengths with slot reuse.""
 import pytest
 import torch
 
-from helpers import CONFIGS, TOL, max_err, model_folder, plain_logits, tokens_for
+from helpers import TOL, max_err, model_folder, plain_logits, tokens_for
 
 pytestmark = pytest.mark.gpu
 

@@ -10,7 +10,7 @@ import torch
 import torch.nn.functional as F
 
 import plain_llama as P
-from helpers import TINY_A, TINY_B, model_folder
+from helpers import model_folder
 
 torch.manual_seed(0)
 D64 = torch.float64
