@@ -31,7 +31,7 @@ def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     rows, n_in = x.shape
     n_out = w.shape[0]
     assert w.shape[1] == n_in
-    y = torch.zeros(rows, n_out, dtype=x.dtype)
+    y = torch.zeros(rows, n_out, dtype=x.dtype, device=x.device)
     for r in range(rows):
         y[r] = (w * x[r][None, :]).sum(dim=1)
     return y
@@ -153,7 +153,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_head: int, n_
     d = q.shape[1] // n_head
     n_rep = n_head // n_kv
     scale = 1.0 / math.sqrt(d)
-    out = torch.zeros(t_len, n_head * d, dtype=q.dtype)
+    out = torch.zeros(t_len, n_head * d, dtype=q.dtype, device=q.device)
     for pos in range(t_len):
         lo = 0 if window is None else max(0, pos - window + 1)
         for qh in range(n_head):
@@ -179,9 +179,10 @@ def swiglu(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: to
 class PlainLlama:
     """config.json + tensors by name -> logits of whole sequences."""
 
-    def __init__(self, config: dict, tensors: dict, dtype=torch.float64):
+    def __init__(self, config: dict, tensors: dict, dtype=torch.float64, device="cpu"):
         c = config
         self.dtype = dtype
+        self.device = device        # where the sums run; the element-by-element rotation stays on the host
         self.n_embd = int(c["hidden_size"])
         self.n_layer = int(c["num_hidden_layers"])
         self.n_head = int(c["num_attention_heads"])
@@ -196,15 +197,15 @@ class PlainLlama:
         self.tied = bool(c.get("tie_word_embeddings", False))
         self.window = c.get("sliding_window")
         self.inv_freq = rope_inv_freq(self.head_dim, self.theta, self.scaling)
-        self.w = {k: v.to(dtype) for k, v in tensors.items()}
+        self.w = {k: v.to(device=device, dtype=dtype) for k, v in tensors.items()}
 
     @classmethod
-    def from_folder(cls, folder: str, dtype=torch.float64) -> "PlainLlama":
+    def from_folder(cls, folder: str, dtype=torch.float64, device="cpu") -> "PlainLlama":
         from safetensors.torch import load_file
         with open(os.path.join(folder, "config.json")) as f:
             config = json.load(f)
         tensors = load_file(os.path.join(folder, "model.safetensors"))
-        return cls(config, tensors, dtype)
+        return cls(config, tensors, dtype, device)
 
     def layer(self, x: torch.Tensor, il: int) -> torch.Tensor:
         """One block: norm, q/k/v, rotate q and k, attention, output projection
@@ -216,11 +217,13 @@ class PlainLlama:
         q = linear(h, w[p + "self_attn.q_proj.weight"])
         k = linear(h, w[p + "self_attn.k_proj.weight"])
         v = linear(h, w[p + "self_attn.v_proj.weight"])
+        q, k = q.cpu(), k.cpu()
         for pos in range(x.shape[0]):
             for hh in range(self.n_head):
                 q[pos, hh * d:(hh + 1) * d] = rope(q[pos, hh * d:(hh + 1) * d], pos, self.inv_freq, self.style)
             for hh in range(self.n_kv):
                 k[pos, hh * d:(hh + 1) * d] = rope(k[pos, hh * d:(hh + 1) * d], pos, self.inv_freq, self.style)
+        q, k = q.to(x.device), k.to(x.device)
         a = attention(q, k, v, self.n_head, self.n_kv, self.window)
         x = x + linear(a, w[p + "self_attn.o_proj.weight"])
         h2 = rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps)

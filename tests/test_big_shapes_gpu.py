@@ -1,7 +1,7 @@
 """The kernels that only wide models select (256 x 256 tiles, the token-resident and the
-panel products, 8-wave flash attention, decode splits) at the widths of Llama-3-8B with two
-layers: the bfloat16 engine's prompt step, decode steps and a mid-size batch against the
-float32 engine, which runs the generic kernels only."""
+panel products, flash attention over many blocks, decode splits) at the widths of Llama-3-8B
+with two layers: the float32 engine against the plain implementation, and the bfloat16
+engine's prompt step, decode steps and a mid-size batch against the float32 engine."""
 import numpy as np
 import pytest
 import torch
@@ -27,6 +27,32 @@ def folder(tmp_path_factory):
 
 def _rel(a, b):
     return float((a.double() - b.double()).abs().max() / b.double().abs().max())
+
+
+def test_wide_model_float32_against_plain(folder):
+    """The float32 engine at full width (sums over 4,096 and 14,336 terms, a vocabulary of
+    128,256) against the plain implementation in float64, whose sums run on the GPU for their
+    size: a prompt in one step, then tokens one by one."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(__file__))
+    import rbitnet_amd
+    from plain_llama import PlainLlama
+    rng = np.random.default_rng(11)
+    tokens = [int(t) for t in rng.integers(0, 128256, size=40)]
+    plain = PlainLlama.from_folder(folder, device="cuda:0")
+    want = plain.logits(tokens).cpu()
+    del plain
+    torch.cuda.empty_cache()
+    eng = rbitnet_amd.Engine.load_path(folder, dtype="float32", max_tokens=64, max_batch=1)
+    slot = eng.alloc_slot()
+    got = [eng.step([(slot, tokens[:34])], "all")]
+    for t in tokens[34:]:
+        got.append(eng.step([(slot, [t])], "last"))
+    eng.free_slot(slot)
+    got = torch.cat(got).cpu()
+    assert got.shape == want.shape
+    assert _rel(got, want) < 2e-5
 
 
 def test_wide_model_bfloat16_against_float32(folder):
