@@ -202,6 +202,12 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
     };
 #pragma unroll
     for (int u = 0; u < U; ++u) load_stage(u, u);
+    // the sums of squares were asked for before the first stage and arrive before it: added up
+    // here, they do not occupy registers during the loop
+    if (SCALED) {
+#pragma unroll
+      for (int cb = 0; cb < MB; ++cb) ss[cb] = squares_sum(asked[cb]);
+    }
     for (int s0 = 0; s0 + U < stages; s0 += U) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -212,6 +218,10 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
 #pragma unroll
     for (int u = 0; u < U; ++u) multiply_stage(u);
   } else {
+    if (SCALED) {
+#pragma unroll
+      for (int cb = 0; cb < MB; ++cb) ss[cb] = squares_sum(asked[cb]);
+    }
     for (int k0 = k_begin; k0 < k_end; k0 += 128) {
       Frag8 a[R][4], b[MB][4];
 #pragma unroll
@@ -236,7 +246,6 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
   if (SCALED) {
 #pragma unroll
     for (int cb = 0; cb < MB; ++cb) {
-      ss[cb] = squares_sum(asked[cb]);
       ss[cb] += __shfl_xor(ss[cb], 16, RB_WAVE);
       ss[cb] += __shfl_xor(ss[cb], 32, RB_WAVE);
     }
@@ -364,11 +373,21 @@ static int dispatch_skinny(const GemmTokens& x, const bf16_t* w, void* c, const 
   const int mb = (m + 15) / 16;
   RB_REQUIRE(!FOLDS || mb == 1, "rb_gemm_bf16: a product that folds its neighbours in takes at most 16 tokens, not %d",
              m);
-  // rows of W per wave: more of them reuse the token operand better, fewer give more
-  // workgroups; keep at least about two workgroups per compute unit
+  // Row tiles of W per wave (16 R rows per workgroup): more of them reuse the token operand
+  // better, fewer deal the rows to the 256 compute units more evenly.  The time goes with the
+  // rows that the busiest compute unit gets, at a price per row that falls with R (measured:
+  // about 15 % / R).  57344 rows at K = 8192: R = 4 gives 896 workgroups, 4 on some compute
+  // units and 3 on others, 194 us; R = 2 gives every one 7: 175 us.
   int r = 1;
-  if (n >= 16384) r = 4;
-  else if (n >= 6144) r = 2;
+  double best = 0.0;
+  for (int cand = (EPI == 1 ? 2 : 1); cand <= 4; cand *= 2) {
+    const long long wgs = (n + 16 * cand - 1) / (16 * cand);
+    const double cost = (double)((wgs + 255) / 256 * 16 * cand) * (1.0 + 0.15 / cand);
+    if (best == 0.0 || cost <= best) {
+      best = cost;
+      r = cand;
+    }
+  }
   if (g_tune_r) r = g_tune_r;
   if (EPI == 1 && r < 2) r = 2;
 #define RB_SK(MBV, RV) return launch_skinny_u<MBV, RV, EPI, TO, SCALED>(x, w, c, after, m, n, k, s)
