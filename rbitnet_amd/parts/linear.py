@@ -12,6 +12,7 @@ between them; otherwise the caller is left with the sum and the rows are normali
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -26,10 +27,14 @@ def uses_matrix_cores(dtype: torch.dtype, k: int) -> bool:
     return dtype == torch.bfloat16 and k % 8 == 0
 
 
+# RBITNET_FOLD=0 (measurements only): sums and norms stay kernels of their own
+_FOLD = os.environ.get("RBITNET_FOLD", "1") != "0"
+
+
 def _few(lib, x, w: torch.Tensor) -> bool:
     """Whether the kernel for a few tokens, which folds its neighbours in, takes this product."""
     m, k = x.shape
-    return uses_matrix_cores(x.dtype, k) and lib.gemm_bf16_few_ok(m, w.shape[0], k)
+    return _FOLD and uses_matrix_cores(x.dtype, k) and lib.gemm_bf16_few_ok(m, w.shape[0], k)
 
 
 def _from_gained(lib, x: GainedRows, w: torch.Tensor, out: torch.Tensor, epilogue: int) -> None:
