@@ -663,6 +663,35 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
   const int first_page = lo / RB_PAGE, last_page = pos / RB_PAGE;
   const int32_t* pages = block_table + (size_t)b * bt_stride;
 
+  // ---- A page's way from memory (its number in the table, then its rows) is the longest wait
+  // of a short step, so it starts early: the numbers of the wave's first two pages are asked
+  // for here, the first page's values and keys as soon as q has been prepared (before the
+  // barrier), every further page's keys while the page before is worked on, and its number a
+  // page before that.
+  Frag8 kf[4][KS], kf_next[4][KS];
+  const int pg_step = NW * n_splits;
+  const int pg_first = first_page + split + n_splits * wave;
+  int id_next = pg_first <= last_page ? pages[pg_first] : 0;                       // the page worked on next
+  int id_after = pg_first + pg_step <= last_page ? pages[pg_first + pg_step] : 0;  // the one after it
+  uint16_t* vpage = vpages + wave * RB_PAGE * D;
+  const uint32_t vpage_lds = (uint32_t)(uintptr_t)vpage;
+  auto ask_values = [&](int page) {        // into this wave's area of LDS
+    const bf16_t* rows = v_pages + ((size_t)page * n_kv + kvh) * RB_PAGE * D;
+#pragma unroll
+    for (int i = 0; i < VI; ++i) {
+      const int key = i * RPI + lane / CPR;
+      const int chunk = (lane % CPR) ^ v_swizzle<D>(key);
+      load_to_lds16(rows, (uint32_t)(key * D + chunk * 8) * 2u, vpage_lds + i * 1024u);
+    }
+  };
+  auto ask_keys = [&](int page) {          // into kf_next
+    const bf16_t* rows = k_pages + ((size_t)page * n_kv + kvh) * RB_PAGE * D;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int st = 0; st < KS; ++st) kf_next[t][st].u = load16(rows + (size_t)(16 * t + c16) * D + 32 * st + 8 * grp);
+  };
+
   // ---- q of the group (rotated here when FUSED) as bfloat16 rows in LDS, zero rows beyond it
   if (FUSED) {
     const int row_width = (n_heads + 2 * n_kv) * D;
@@ -697,6 +726,12 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
       q_h[idx] = gg < G ? q_in[((size_t)b * n_heads + kvh * G + gg) * D + d].bits : (uint16_t)0;
     }
   }
+  int page_cur = 0;
+  if (pg_first <= last_page) {
+    page_cur = __builtin_amdgcn_readfirstlane(id_next);
+    ask_values(page_cur);
+    ask_keys(page_cur);
+  }
   __syncthreads();
   if (FUSED && split == (last_page - first_page) % n_splits) {      // this workgroup owns the last page
     const int page = pages[last_page];
@@ -714,25 +749,33 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
   f32x4_t acc_o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) acc_o[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  uint16_t* vpage = vpages + wave * RB_PAGE * D;
-  const uint32_t vpage_lds = (uint32_t)(uintptr_t)vpage;
 
-  for (int pg = first_page + split + n_splits * wave; pg <= last_page; pg += NW * n_splits) {
-    const int page = __builtin_amdgcn_readfirstlane(pages[pg]);
-    const size_t base = ((size_t)page * n_kv + kvh) * RB_PAGE * D;
-    // the reads of the previous page have all returned before its area is overwritten
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int i = 0; i < VI; ++i) {
-      const int key = i * RPI + lane / CPR;
-      const int chunk = (lane % CPR) ^ v_swizzle<D>(key);
-      load_to_lds16(v_pages + base, (uint32_t)(key * D + chunk * 8) * 2u, vpage_lds + i * 1024u);
-    }
-    Frag8 kf[4][KS];
+  for (int pg = pg_first; pg <= last_page; pg += pg_step) {
+    // This page's keys must all have arrived here, before the loads into LDS below are issued:
+    // the compiler does not see those (they are assembly) and would count them out wrongly if
+    // it waited for keys later.  Touching every register makes it wait now.
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int st = 0; st < KS; ++st) kf[t][st].u = load16(k_pages + base + (size_t)(16 * t + c16) * D + 32 * st + 8 * grp);
+      for (int st = 0; st < KS; ++st) {
+        kf[t][st] = kf_next[t][st];
+        asm volatile("" ::"v"(kf[t][st].u.x), "v"(kf[t][st].u.y), "v"(kf[t][st].u.z), "v"(kf[t][st].u.w) : "memory");
+      }
+    if (pg != pg_first) {
+      // the reads of the previous page have all returned before its area is overwritten (the
+      // first page's values were asked for before the barrier)
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      ask_values(page_cur);
+    }
+    // the next page's keys (its number was asked for a page ago), and the number of the one after
+    const bool more = pg + pg_step <= last_page;
+    const bool more2 = pg + 2 * pg_step <= last_page;
+    int page_nx = 0;
+    if (more) {
+      page_nx = __builtin_amdgcn_readfirstlane(id_after);
+      ask_keys(page_nx);
+      if (more2) id_after = pages[pg + 2 * pg_step];
+    }
     if (FUSED && pg == last_page) {
       // the token's own key is not in the cache yet (or only just): take it from LDS
       const int t_new = (pos % RB_PAGE) / 16, r_new = pos % 16;
@@ -788,8 +831,11 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
       pf[s2].u.z = pack_bf16x2(sc[2 * s2 + 1][0], sc[2 * s2 + 1][1]);
       pf[s2].u.w = pack_bf16x2(sc[2 * s2 + 1][2], sc[2 * s2 + 1][3]);
     }
-    // ---- the page of V has arrived (loads complete in issue order, and K came after it)
-    wait_vm<0>();
+    // ---- the page of V has arrived (loads complete in issue order; the next page's keys,
+    // asked for after it, may still be on their way)
+    if (more2) wait_vm<4 * KS + 1>();
+    else if (more) wait_vm<4 * KS>();
+    else wait_vm<0>();
     if (pg == last_page) {
       const int r_pos = pos % RB_PAGE;
       for (int row = FUSED ? r_pos : r_pos + 1; row < RB_PAGE; ++row) {
@@ -829,6 +875,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
         acc_o[dt] = mfma16(vf, pf[s2], acc_o[dt]);
       }
     }
+    page_cur = page_nx;
   }
 
   // ---- the waves' states into one (the pages' area is reused for the outputs)
