@@ -34,8 +34,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
   constexpr int DC = D / 8;           // 16-byte chunks per row
   constexpr int NT = 64 * NW;
   constexpr int KCH = RB_PAGE * DC / NT;
-  __shared__ __attribute__((aligned(16))) bf16_t ks[RB_PAGE * KLD];
-  __shared__ __attribute__((aligned(16))) bf16_t vt[D * VLD];
+  // two tiles of each: the next one is written while the current one is read
+  __shared__ __attribute__((aligned(16))) bf16_t ks2[2][RB_PAGE * KLD];
+  __shared__ __attribute__((aligned(16))) bf16_t vt2[2][D * VLD];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, g = lane >> 5;
@@ -132,7 +133,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
       }
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](int buf) {
+    bf16_t* ks = ks2[buf];
+    bf16_t* vt = vt2[buf];
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
       const int c = tid + NT * i;
@@ -165,13 +168,19 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     }
   };
 
+  // Tile kt is read from buffer (kt - first_tile) % 2 while tile kt + 1 comes from memory into
+  // registers and, after the products, goes into the other buffer: one barrier a tile, behind
+  // which everyone has finished reading what the tile after next will overwrite.
   load_tile(first_tile);
+  store_tile(0);
+  __syncthreads();
   for (int kt = first_tile; kt <= last_tile; ++kt) {
-    __syncthreads();                 // everyone is done reading the previous tile
-    store_tile();
-    __syncthreads();
-    if (kt + 1 <= last_tile) load_tile(kt + 1);
-    if (!(wave_on && kt >= wave_first && kt <= wave_last)) continue;
+    const int buf = (kt - first_tile) & 1;
+    const bf16_t* ks = ks2[buf];
+    const bf16_t* vt = vt2[buf];
+    const bool next = kt + 1 <= last_tile;
+    if (next) load_tile(kt + 1);
+    if (wave_on && kt >= wave_first && kt <= wave_last) {
 
     // ---- S^T = K Q^T: rows keys, columns queries
     f32x16_t sacc[2];
@@ -249,6 +258,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
           oacc[i] = mfma32(a, pb, oacc[i]);
         }
       }
+    }
+    if (next) store_tile(buf ^ 1);
+    __syncthreads();
   }
 
   if (!wave_on || !q_ok) return;
