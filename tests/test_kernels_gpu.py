@@ -304,9 +304,9 @@ def test_attention_prefill_bf16(lib, n_heads, n_kv, d, window):
     assert _rel(out, want) < 1.5e-2
 
 
-@pytest.mark.parametrize("waves", [0, 8])
+@pytest.mark.parametrize("waves", [0, 4, 8])
 @pytest.mark.parametrize("n_heads,n_kv,d,t,window", [(24, 24, 64, 1536, 0), (32, 8, 128, 1100, 0), (8, 2, 128, 2500, 300),
-                                                    (4, 4, 64, 700, 0)])
+                                                    (4, 4, 64, 700, 0), (6, 3, 128, 333, 70)])
 def test_attention_prefill_of_a_long_prompt(lib, waves, n_heads, n_kv, d, t, window):
     """One prompt of a thousand tokens and more, where the order in which the workgroups take
     the blocks of queries matters: between 257 and 512 workgroups a sequence (288, 280 and 316
