@@ -430,8 +430,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       float y0 = x0, y1 = x1;
       if (cr) {
         const float c = cr[i], sn = sr[i];
-        y0 = x0 * c - x1 * sn;
-        y1 = x0 * sn + x1 * c;
+        rotate_pair(x0, x1, c, sn, y0, y1);
       }
       uint16_t* dst = gg < G ? q_h[gg] : knew_h;
       dst[i0] = f32_to_bf16_bits(y0);
@@ -724,8 +723,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
       float y0 = x0, y1 = x1;
       if (cr) {
         const float c = cr[i], sn = sr[i];
-        y0 = x0 * c - x1 * sn;
-        y1 = x0 * sn + x1 * c;
+        rotate_pair(x0, x1, c, sn, y0, y1);
       }
       dst[i0] = f32_to_bf16_bits(y0);
       dst[i1] = f32_to_bf16_bits(y1);

@@ -76,6 +76,15 @@ struct Num<bf16_t> {
   static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 };
 
+// ---------------------------------------------------------------- rotation of a pair
+// (x0, x1) turned by the angle whose cosine and sine are c and s (llama/model.rs:122-136). The
+// operations are spelled out so that every kernel that rotates rounds the same way, whatever
+// the compiler would have contracted: the same q, k and logits whichever kernel rotated them.
+__device__ __forceinline__ void rotate_pair(float x0, float x1, float c, float s, float& y0, float& y1) {
+  y0 = __fmaf_rn(x0, c, -__fmul_rn(x1, s));
+  y1 = __fmaf_rn(x0, s, __fmul_rn(x1, c));
+}
+
 // ---------------------------------------------------------------- terms of a product
 // A product whose K was cut into slices may be left as its slices' sums, `stride` floats
 // apart: p[0] + p[stride] + ... in that order (the order in which the product's own kernel

@@ -239,8 +239,7 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int n_terms,
     float y0 = x0, y1 = x1;
     if (cr) {
       const float c = cr[i], s = sr[i];
-      y0 = x0 * c - x1 * s;
-      y1 = x0 * s + x1 * c;
+      rotate_pair(x0, x1, c, s, y0, y1);
     }
     if (h < n_heads) {
       TC* dst = q_out + ((size_t)t * n_heads + h) * head_dim;
