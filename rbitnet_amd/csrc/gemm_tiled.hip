@@ -309,79 +309,103 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   };
 
   // ---- fragments: row base + 32 i + l32, chunk 2 ks + g, found in slot chunk ^ swz(l32)
+  constexpr int KSTEPS = BK / 16;
+  static_assert(KSTEPS % 2 == 0, "the fragment buffers alternate by depth step");
   const int sw = (l32 / RPB) % CPR;
   const bf16_t* wfrag = lds + (size_t)(wn0 + l32) * BK;
   const bf16_t* xfrag = lds + (size_t)BN * BK + (size_t)(wm0 + l32) * BK;
-  auto multiply = [&](int kt) {
+  Frag8 a[2][TN], b[2][TM];
+  auto load_frags = [&](int buf2, int kt, int ks) {
     const bf16_t* wb = wfrag + (size_t)(kt % S) * STAGE;
     const bf16_t* xb = xfrag + (size_t)(kt % S) * STAGE;
-    Frag8 a[2][TN], b[2][TM];
-    auto load_frags = [&](int buf2, int ks) {
-      const int slot = ((2 * ks + g) ^ sw) * 8;
+    const int slot = ((2 * ks + g) ^ sw) * 8;
 #pragma unroll
-      for (int i = 0; i < TN; ++i) a[buf2][i].u = *reinterpret_cast<const uint4*>(wb + 32 * i * BK + slot);
+    for (int i = 0; i < TN; ++i) a[buf2][i].u = *reinterpret_cast<const uint4*>(wb + 32 * i * BK + slot);
 #pragma unroll
-      for (int j = 0; j < TM; ++j) b[buf2][j].u = *reinterpret_cast<const uint4*>(xb + 32 * j * BK + slot);
-    };
-    load_frags(0, 0);
+    for (int j = 0; j < TM; ++j) b[buf2][j].u = *reinterpret_cast<const uint4*>(xb + 32 * j * BK + slot);
+  };
+  // the tokens are the MFMA's rows and W's rows its columns: a lane then holds one column of W's
+  // rows for 16 tokens, and a wave's store covers 32 consecutive outputs of a token
+  auto mfmas = [&](int buf2) {
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      if (ks + 1 < BK / 16) load_frags((ks + 1) & 1, ks + 1);
+    for (int i = 0; i < TN; ++i)
 #pragma unroll
-      for (int i = 0; i < TN; ++i)
+      for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(b[buf2][j], a[buf2][i], acc[i][j]);
+  };
+
+  // ---- main loop.  The barrier that hands over tile kt + 1 stands before the last depth step
+  // of tile kt, whose fragments are in registers by then: its MFMAs run while the first
+  // fragments of tile kt + 1 come from LDS and while the other waves arrive, and the stage of
+  // tile kt is free for tile kt + S from there on.
 #pragma unroll
-        for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[ks & 1][i], b[ks & 1][j], acc[i][j]);
+  for (int s = 0; s < S; ++s)
+    if (s < k_tiles) issue(s);
+  if (S - 1 < k_tiles) wait_vm<LOADS * (S - 1)>();
+  else wait_vm<0>();
+  __syncthreads();
+  load_frags(0, 0, 0);
+  auto steps_but_last = [&](int kt) {
+#pragma unroll
+    for (int ks = 0; ks + 1 < KSTEPS; ++ks) {
+      load_frags((ks + 1) & 1, kt, ks + 1);
+      mfmas(ks & 1);
     }
     // the order the scheduler is asked to keep: the fragments of depth step ks + 1 are all
     // requested before the MFMAs of step ks, which then cover the LDS latency
-    constexpr int KSTEPS = BK / 16;
-    __builtin_amdgcn_sched_group_barrier(0x100, TN + TM, 0);
 #pragma unroll
     for (int ks = 0; ks + 1 < KSTEPS; ++ks) {
       __builtin_amdgcn_sched_group_barrier(0x100, TN + TM, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, TN * TM, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, TN * TM, 0);
   };
-
-#pragma unroll
-  for (int s = 0; s < S - 1; ++s)
-    if (s < k_tiles) issue(s);
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    // tile kt must have landed; in the steady state the S - 2 tiles after it stay in flight
-    if (kt + S - 2 < k_tiles) wait_vm<LOADS * (S - 2)>();
-    else wait_vm<0>();
-    __syncthreads();                  // everyone's part of tile kt is in LDS, and tile kt - 1 has been read by all
-    if (kt + S - 1 < k_tiles) issue(kt + S - 1);      // into the stage tile kt - 1 occupied
-    multiply(kt);
+  for (int kt = 0; kt + 1 < k_tiles; ++kt) {
+    steps_but_last(kt);
+    // tile kt + 1 must have landed; in the steady state the S - 2 tiles after it stay in flight
+    if (S == 2 || kt + S - 1 >= k_tiles) wait_vm<0>();
+    else wait_vm<LOADS * (S - 2)>();
+    // the last fragments of tile kt are in registers before anyone may overwrite its stage
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();                  // everyone's part of tile kt + 1 is in LDS, and nobody reads tile kt's stage any more
+    if (kt + S < k_tiles) issue(kt + S);
+    load_frags(0, kt + 1, 0);
+    mfmas((KSTEPS - 1) & 1);
   }
+  steps_but_last(k_tiles - 1);
+  mfmas((KSTEPS - 1) & 1);
 
-  // ---- lane holds, per (i, j): token m0 + wm0 + 32 j + l32, W rows base + 8 (e / 4) + 4 g + e % 4
+  // ---- lane holds, per (i, j): W row n0 + wn0 + 32 i + l32, tokens base + 8 (e / 4) + 4 g + e % 4
 #pragma unroll
   for (int i = 0; i < TN; ++i)
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
-      const int mm = m0 + wm0 + 32 * j + l32;
-      if (mm >= m) continue;
-      const int nbase = n0 + wn0 + 32 * i;
+      const int nn = n0 + wn0 + 32 * i + l32;
+      const int mbase = m0 + wm0 + 32 * j + 4 * g;
       if (EPI == 0) {
+        if (nn >= n) continue;
         // a slice of K: partial sums go to this slice's [M, N] slab, to be added up in a fixed order
-        float* slab = slabs ? slabs + ((size_t)blockIdx.y * m + mm) * n : nullptr;
-        TO* dst = c + (size_t)mm * n;
+        float* slab = slabs ? slabs + (size_t)blockIdx.y * m * n + nn : nullptr;
+        TO* dst = c + nn;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const int nn = nbase + 8 * (e / 4) + 4 * g + (e % 4);
-          if (nn >= n) continue;
-          if (slab) slab[nn] = acc[i][j][e];
-          else Num<TO>::store(dst + nn, acc[i][j][e]);
+          const int mm = mbase + 8 * (e / 4) + (e % 4);
+          if (mm >= m) continue;
+          if (slab) slab[(size_t)mm * n] = acc[i][j][e];
+          else Num<TO>::store(dst + (size_t)mm * n, acc[i][j][e]);
         }
       } else {
+        // gate rows in lanes 0..15 of a half wave, up rows in lanes 16..31: the two halves swap what
+        // the other needs, the lower one finishing the even tokens and the upper one the odd ones
         const int half_n = n / 2;
-        TO* dst = c + (size_t)mm * half_n;
+        const bool upper = (l32 & 16) != 0;
+        const int col = (n0 + wn0 + 32 * i) / 2 + (l32 & 15);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int nn = nbase / 2 + 8 * (e / 4) + 4 * g + (e % 4);
-          if (nn < half_n) Num<TO>::store(dst + nn, silu_f32(acc[i][j][e]) * acc[i][j][e + 8]);
+        for (int e = 0; e < 16; e += 2) {
+          const float mine = upper ? acc[i][j][e + 1] : acc[i][j][e];
+          const float give = upper ? acc[i][j][e] : acc[i][j][e + 1];
+          const float got = __shfl_xor(give, 16);
+          const int mm = mbase + 8 * (e / 4) + (e % 4) + (upper ? 1 : 0);
+          const float gate = upper ? got : mine, up = upper ? mine : got;
+          if (mm < m && col < half_n) Num<TO>::store(c + (size_t)mm * half_n + col, silu_f32(gate) * up);
         }
       }
     }
