@@ -1,6 +1,6 @@
 // Products with many tokens (prefill) and with 17..64 tokens: tiles of W and of the tokens
-// through LDS, MFMA 32x32x16 bf16, float32 accumulation.  W rows are the row operand of the
-// MFMA and the tokens its columns.
+// through LDS, MFMA 32x32x16 bf16, float32 accumulation.  The tokens are the row operand of the
+// MFMA and W's rows its columns, so that the lanes of a wave hold consecutive outputs of a token.
 //
 // Epilogue 1 expects W with gate and up rows interleaved in blocks of 16 and writes
 // silu(gate) * up (llama/model.rs:297-302 of the reference) instead of the two products.
@@ -38,6 +38,41 @@ __device__ __forceinline__ bool tile_of_workgroup(int m_tiles, int n_tiles, int*
   *mt = first_m + r % rows;
   *nt = r / rows;
   return true;
+}
+
+// What a lane holds of a 32 x 32 piece when the tokens were the MFMA's rows and W's rows its
+// columns: W row first_row + l32 for the 16 tokens mbase + 8 (e / 4) + e % 4 (mbase includes the
+// lane's 4 g).  A wave's store then covers 32 consecutive outputs of each of two tokens.  With
+// `slab`, the sums go to that slice's [M, N] slab instead, to be added up later in a fixed order.
+template <int EPI, typename TO>
+__device__ __forceinline__ void store_piece(const f32x16_t& acc, TO* __restrict__ c, float* __restrict__ slab,
+                                            int first_row, int l32, int mbase, int m, int n) {
+  if (EPI == 0) {
+    const int nn = first_row + l32;
+    if (nn >= n) return;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int mm = mbase + 8 * (e / 4) + (e % 4);
+      if (mm >= m) continue;
+      if (slab) slab[(size_t)mm * n + nn] = acc[e];
+      else Num<TO>::store(c + (size_t)mm * n + nn, acc[e]);
+    }
+  } else {
+    // gate rows in lanes 0..15 of a half wave, up rows in lanes 16..31: the two halves swap what
+    // the other needs, the lower one finishing the even tokens and the upper one the odd ones
+    const int half_n = n / 2;
+    const bool upper = (l32 & 16) != 0;
+    const int col = first_row / 2 + (l32 & 15);
+#pragma unroll
+    for (int e = 0; e < 16; e += 2) {
+      const float mine = upper ? acc[e + 1] : acc[e];
+      const float give = upper ? acc[e] : acc[e + 1];
+      const float got = __shfl_xor(give, 16);
+      const int mm = mbase + 8 * (e / 4) + (e % 4) + (upper ? 1 : 0);
+      const float gate = upper ? got : mine, up = upper ? mine : got;
+      if (mm < m && col < half_n) Num<TO>::store(c + (size_t)mm * half_n + col, silu_f32(gate) * up);
+    }
+  }
 }
 
 #define TG_BK 64
@@ -146,7 +181,7 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_tiled_kernel(
 #pragma unroll
         for (int i = 0; i < TN; ++i)
 #pragma unroll
-          for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[ks & 1][i], b[ks & 1][j], acc[i][j]);
+          for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(b[ks & 1][j], a[ks & 1][i], acc[i][j]);
       }
     } else {
       // 8 waves: two per SIMD cover each other's LDS latency, and registers are scarce
@@ -162,7 +197,7 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_tiled_kernel(
 #pragma unroll
         for (int i = 0; i < TN; ++i)
 #pragma unroll
-          for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+          for (int j = 0; j < TM; ++j) acc[i][j] = mfma32(b[j], a[i], acc[i][j]);
       }
     }
   };
@@ -194,31 +229,12 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_tiled_kernel(
     }
   }
 
-  // ---- lane holds, per (i, j): token m0 + wm0 + 32 j + l32, W rows base + 8 (e / 4) + 4 g + e % 4
+  // ---- lane holds, per (i, j): W row n0 + wn0 + 32 i + l32, tokens base + 8 (e / 4) + 4 g + e % 4
 #pragma unroll
   for (int i = 0; i < TN; ++i)
 #pragma unroll
-    for (int j = 0; j < TM; ++j) {
-      const int mm = m0 + wm0 + 32 * j + l32;
-      if (mm >= m) continue;
-      const int nbase = n0 + wn0 + 32 * i;
-      if (EPI == 0) {
-        TO* dst = c + (size_t)mm * n;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int nn = nbase + 8 * (e / 4) + 4 * g + (e % 4);
-          if (nn < n) Num<TO>::store(dst + nn, acc[i][j][e]);
-        }
-      } else {
-        const int half_n = n / 2;
-        TO* dst = c + (size_t)mm * half_n;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int nn = nbase / 2 + 8 * (e / 4) + 4 * g + (e % 4);
-          if (nn < half_n) Num<TO>::store(dst + nn, silu_f32(acc[i][j][e]) * acc[i][j][e + 8]);
-        }
-      }
-    }
+    for (int j = 0; j < TM; ++j)
+      store_piece<EPI, TO>(acc[i][j], c, nullptr, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -374,41 +390,12 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   mfmas((KSTEPS - 1) & 1);
 
   // ---- lane holds, per (i, j): W row n0 + wn0 + 32 i + l32, tokens base + 8 (e / 4) + 4 g + e % 4
+  float* slab = slabs ? slabs + (size_t)blockIdx.y * m * n : nullptr;      // this slice of K's partial sums
 #pragma unroll
   for (int i = 0; i < TN; ++i)
 #pragma unroll
-    for (int j = 0; j < TM; ++j) {
-      const int nn = n0 + wn0 + 32 * i + l32;
-      const int mbase = m0 + wm0 + 32 * j + 4 * g;
-      if (EPI == 0) {
-        if (nn >= n) continue;
-        // a slice of K: partial sums go to this slice's [M, N] slab, to be added up in a fixed order
-        float* slab = slabs ? slabs + (size_t)blockIdx.y * m * n + nn : nullptr;
-        TO* dst = c + nn;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int mm = mbase + 8 * (e / 4) + (e % 4);
-          if (mm >= m) continue;
-          if (slab) slab[(size_t)mm * n] = acc[i][j][e];
-          else Num<TO>::store(dst + (size_t)mm * n, acc[i][j][e]);
-        }
-      } else {
-        // gate rows in lanes 0..15 of a half wave, up rows in lanes 16..31: the two halves swap what
-        // the other needs, the lower one finishing the even tokens and the upper one the odd ones
-        const int half_n = n / 2;
-        const bool upper = (l32 & 16) != 0;
-        const int col = (n0 + wn0 + 32 * i) / 2 + (l32 & 15);
-#pragma unroll
-        for (int e = 0; e < 16; e += 2) {
-          const float mine = upper ? acc[i][j][e + 1] : acc[i][j][e];
-          const float give = upper ? acc[i][j][e] : acc[i][j][e + 1];
-          const float got = __shfl_xor(give, 16);
-          const int mm = mbase + 8 * (e / 4) + (e % 4) + (upper ? 1 : 0);
-          const float gate = upper ? got : mine, up = upper ? mine : got;
-          if (mm < m && col < half_n) Num<TO>::store(c + (size_t)mm * half_n + col, silu_f32(gate) * up);
-        }
-      }
-    }
+    for (int j = 0; j < TM; ++j)
+      store_piece<EPI, TO>(acc[i][j], c, slab, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n);
 }
 
 template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO>
