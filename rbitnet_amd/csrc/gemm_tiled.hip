@@ -374,20 +374,60 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
       __builtin_amdgcn_sched_group_barrier(0x008, TN * TM, 0);
     }
   };
-  for (int kt = 0; kt + 1 < k_tiles; ++kt) {
-    steps_but_last(kt);
+  // One load of tile kt (number l of the LOADS a wave has), one fragment of a depth step.
+  auto issue_one = [&](int kt, int l) {
+    const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
+    const uint32_t kbytes = (uint32_t)(kt0 + kt) * (BK * 2);
+    if (l < W_LOADS) load_to_lds16(wtile, woff[l] + kbytes, stage + (uint32_t)(wave + NWAVES * l) * 1024u);
+    else
+      load_to_lds16(xtile, xoff[l - W_LOADS] + kbytes,
+                    stage + (uint32_t)(BN * BK * 2) + (uint32_t)(wave + NWAVES * (l - W_LOADS)) * 1024u);
+  };
+  auto frag_one = [&](int buf2, int kt, int ks, int f) {
+    const int slot = ((2 * ks + g) ^ sw) * 8;
+    if (f < TN) a[buf2][f].u = *reinterpret_cast<const uint4*>(wfrag + (size_t)(kt % S) * STAGE + 32 * f * BK + slot);
+    else b[buf2][f - TN].u = *reinterpret_cast<const uint4*>(xfrag + (size_t)(kt % S) * STAGE + 32 * (f - TN) * BK + slot);
+  };
+  // The last depth step of tile kt, behind the barrier: between its MFMAs, one at a time, go the
+  // loads of tile kt + S and the first fragments of tile kt + 1, so that the matrix core never
+  // waits for a run of other instructions (both waves of a SIMD leave the barrier together, and
+  // neither covers the other's).
+  constexpr int NM = TN * TM, LASTBUF = (KSTEPS - 1) & 1;
+  auto last_step = [&](int kt, bool fetch) {
+#pragma unroll
+    for (int q = 0; q < NM; ++q) {
+      acc[q / TM][q % TM] = mfma32(b[LASTBUF][q % TM], a[LASTBUF][q / TM], acc[q / TM][q % TM]);
+      if (fetch) {
+#pragma unroll
+        for (int l = q; l < LOADS; l += NM) issue_one(kt + S, l);
+      }
+#pragma unroll
+      for (int f = q; f < TN + TM; f += NM) frag_one(0, kt + 1, 0, f);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto hand_over = [&](int kt) {
     // tile kt + 1 must have landed; in the steady state the S - 2 tiles after it stay in flight
     if (S == 2 || kt + S - 1 >= k_tiles) wait_vm<0>();
     else wait_vm<LOADS * (S - 2)>();
     // the last fragments of tile kt are in registers before anyone may overwrite its stage
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __syncthreads();                  // everyone's part of tile kt + 1 is in LDS, and nobody reads tile kt's stage any more
-    if (kt + S < k_tiles) issue(kt + S);
-    load_frags(0, kt + 1, 0);
-    mfmas((KSTEPS - 1) & 1);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  int kt = 0;
+  for (; kt + S < k_tiles; ++kt) {
+    steps_but_last(kt);
+    hand_over(kt);
+    last_step(kt, true);
+  }
+  for (; kt + 1 < k_tiles; ++kt) {
+    steps_but_last(kt);
+    hand_over(kt);
+    last_step(kt, false);
   }
   steps_but_last(k_tiles - 1);
-  mfmas((KSTEPS - 1) & 1);
+  mfmas(LASTBUF);
 
   // ---- lane holds, per (i, j): W row n0 + wn0 + 32 i + l32, tokens base + 8 (e / 4) + 4 g + e % 4
   float* slab = slabs ? slabs + (size_t)blockIdx.y * m * n : nullptr;      // this slice of K's partial sums
