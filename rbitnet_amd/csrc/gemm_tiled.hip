@@ -360,20 +360,6 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   else wait_vm<0>();
   __syncthreads();
   load_frags(0, 0, 0);
-  auto steps_but_last = [&](int kt) {
-#pragma unroll
-    for (int ks = 0; ks + 1 < KSTEPS; ++ks) {
-      load_frags((ks + 1) & 1, kt, ks + 1);
-      mfmas(ks & 1);
-    }
-    // the order the scheduler is asked to keep: the fragments of depth step ks + 1 are all
-    // requested before the MFMAs of step ks, which then cover the LDS latency
-#pragma unroll
-    for (int ks = 0; ks + 1 < KSTEPS; ++ks) {
-      __builtin_amdgcn_sched_group_barrier(0x100, TN + TM, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, TN * TM, 0);
-    }
-  };
   // One load of tile kt (number l of the LOADS a wave has), one fragment of a depth step.
   auto issue_one = [&](int kt, int l) {
     const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
@@ -383,16 +369,38 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
       load_to_lds16(xtile, xoff[l - W_LOADS] + kbytes,
                     stage + (uint32_t)(BN * BK * 2) + (uint32_t)(wave + NWAVES * (l - W_LOADS)) * 1024u);
   };
+  // Fragment number f of a depth step, in the order in which the MFMAs first need them:
+  // W's first, all of the tokens', the rest of W's.
   auto frag_one = [&](int buf2, int kt, int ks, int f) {
     const int slot = ((2 * ks + g) ^ sw) * 8;
-    if (f < TN) a[buf2][f].u = *reinterpret_cast<const uint4*>(wfrag + (size_t)(kt % S) * STAGE + 32 * f * BK + slot);
-    else b[buf2][f - TN].u = *reinterpret_cast<const uint4*>(xfrag + (size_t)(kt % S) * STAGE + 32 * (f - TN) * BK + slot);
+    if (f == 0 || f > TM) {
+      const int i = f == 0 ? 0 : f - TM;
+      a[buf2][i].u = *reinterpret_cast<const uint4*>(wfrag + (size_t)(kt % S) * STAGE + 32 * i * BK + slot);
+    } else {
+      b[buf2][f - 1].u = *reinterpret_cast<const uint4*>(xfrag + (size_t)(kt % S) * STAGE + 32 * (f - 1) * BK + slot);
+    }
+  };
+  // A depth step but the last of tile kt: its MFMAs, with the next step's fragments asked for
+  // between them, one after each MFMA, so that a wave keeps the matrix core fed by itself (with
+  // all the reads in a run before the MFMAs, a wave took 27-30 ns per MFMA where the core takes 16-20,
+  // and the two waves of a SIMD, which the barrier keeps in step, did not cover each other).
+  constexpr int NM = TN * TM, LASTBUF = (KSTEPS - 1) & 1;
+  auto steps_but_last = [&](int kt) {
+#pragma unroll
+    for (int ks = 0; ks + 1 < KSTEPS; ++ks) {
+#pragma unroll
+      for (int q = 0; q < NM; ++q) {
+        acc[q / TM][q % TM] = mfma32(b[ks & 1][q % TM], a[ks & 1][q / TM], acc[q / TM][q % TM]);
+#pragma unroll
+        for (int f = q; f < TN + TM; f += NM) frag_one((ks + 1) & 1, kt, ks + 1, f);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
   };
   // The last depth step of tile kt, behind the barrier: between its MFMAs, one at a time, go the
   // loads of tile kt + S and the first fragments of tile kt + 1, so that the matrix core never
   // waits for a run of other instructions (both waves of a SIMD leave the barrier together, and
   // neither covers the other's).
-  constexpr int NM = TN * TM, LASTBUF = (KSTEPS - 1) & 1;
   auto last_step = [&](int kt, bool fetch) {
 #pragma unroll
     for (int q = 0; q < NM; ++q) {
