@@ -568,8 +568,27 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   // unit, 2,048 tokens by 4,096 rows 237 us against 258 at K = 14336 and 82.6 against 83.6 at
   // K = 4096; 1,024 tokens by 6,144 rows 76 against 82; 256 tokens by 28,672 gated rows 80 against
   // 89.  With fewer or more tiles than that they lose (1,024 tokens by 4,096 rows: 204 against 159).
+  // Where they are half or a quarter of a round, K is cut into 2 or 4 slices of at least 32 tiles,
+  // which fills the round again: 512 tokens by 4,096 rows at K = 14336 75 us in 4 slices against 107
+  // in the 64-token tiles (320 tokens: 64 against 106), 1,024 tokens 127 in 2 slices against 146 in
+  // 128 x 128 tiles; at K = 4096, 768 tokens by 4,096 rows 46 against 59, 512 by 6,144 48 against 56.
+  // 160 workgroups of 2 slices still win (640 tokens by 4,096 rows: 43 against 58), 144 do not.
   const long long t256x128 = (long long)((m + 127) / 128) * ((n + 255) / 256);
   if (m > 64 && t256x128 >= 192 && t256x128 <= 256) return {8, 1};
+  if (m > 64 && epilogue == 0) {
+    for (int p = 2; p <= 4; p *= 2)
+      if (t256x128 * p >= 160 && t256x128 * p <= 256 && (k / 64) % p == 0 && k / 64 / p >= 32) return {8, p};
+  }
+  // Between one and two thousand tokens the large tiles are too few for a round by themselves: a deep
+  // product (K >= 8192) is cut into 2 slices of them (1,152 tokens by 4,096 rows at K = 14336: 164 us in
+  // 192 x 256 tiles against 204 in 128 x 128; 1,408 tokens: 182 in 256 x 256 against 208), and where
+  // 192 x 256 tiles alone make most of a round they are taken (1,408 tokens by 6,144 rows: 86 against 110).
+  const long long t192r = (long long)((m + 255) / 256) * ((n + 191) / 192);
+  if (m > 64 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 64) {
+    if (t192r * 2 >= 160 && t192r * 2 <= 256) return {6, 2};
+    if (t256 * 2 >= 160 && t256 * 2 <= 256) return {4, 2};
+  }
+  if (m > 64 && t192r >= 176 && t192r <= 256) return {6, 1};
   if (m > 64 && (t128 >= 256 || m > 512)) return {5, epilogue ? 1 : k_slices(t128, k, 512, k / (4 * m))};
   return {7, epilogue ? 1 : k_slices(t64, k, 256, k / (8 * m))};
 }
