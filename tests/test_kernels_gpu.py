@@ -93,7 +93,10 @@ def test_gemm_bf16_gated(lib, m, ff, k):
                                          (100, 520, 1024, False), (130, 300, 4096, False), (600, 1000, 8192, False),
                                          (300, 4096, 2048, False), (129, 672, 256, True),
                                          (1500, 4000, 256, False), (250, 57344, 64, True), (2048, 4096, 192, False),
-                                         (1030, 14300, 64, False), (1024, 28672 * 2, 64, True)])
+                                         (1030, 14300, 64, False), (1024, 28672 * 2, 64, True),
+                                         (300, 4000, 8192, False), (520, 4100, 4096, False),
+                                         (1100, 4000, 8192, False), (1300, 4096, 8192, False),
+                                         (1300, 6100, 256, False)])
 def test_gemm_bf16_tiles_loaded_straight_into_lds(lib, m, n, k, gated):
     """K a multiple of 64 and more than 64 tokens: the kernels whose tiles go from memory into
     LDS without passing registers, with all three tile sizes (128 x 128; 256 x 256 when its
@@ -103,7 +106,9 @@ def test_gemm_bf16_tiles_loaded_straight_into_lds(lib, m, n, k, gated):
     (64-token tiles in 2 slices at 130 x 300 x 4096, 128 x 128 tiles in 2 at 600 x 1000 x 8192).
     Three cases make 192..256 tiles of 256 rows x 128 tokens, which then run in one round, with
     partial tiles at both edges and the gated epilogue; the last two make fewer rounds of 320-row
-    tiles than of 256-row ones (5 x 45 = 225 against 5 x 56 = 280, and 4 x 180 against 4 x 224)."""
+    tiles than of 256-row ones (5 x 45 = 225 against 5 x 56 = 280, and 4 x 180 against 4 x 224).
+    The last five are tiles too few for a round whose K is cut: 48 tiles of 256 x 128 in 4 slices,
+    85 in 2, 105 tiles of 192 x 256 in 2, 96 of 256 x 256 in 2, and 192 tiles of 192 x 256 uncut."""
     from rbitnet_amd.parts.linear import pack_gate_up
     g = torch.Generator().manual_seed(m + n + k)
     x = torch.randn(m, k, generator=g).bfloat16()
