@@ -438,6 +438,50 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   mfmas(LASTBUF);
 
   // ---- lane holds, per (i, j): W row n0 + wn0 + 32 i + l32, tokens base + 8 (e / 4) + 4 g + e % 4
+  if constexpr (EPI == 1 && sizeof(TO) == 2) {
+    // The gated outputs of a piece are 16 columns wide: stored from the registers, a wave's store
+    // would write 32 bytes of each of four tokens, and the tile's 80 such stores a lane took 27-35 us
+    // of a 320 x 256 tile's 150.  They go through LDS instead (the tiles are done with) and leave
+    // as whole rows of the tile, 16 bytes a lane.
+    constexpr int HC = BN / 2;              // output columns of the tile
+    constexpr int LD = HC + 8;              // 16 bytes of padding: the four tokens of a store hit different banks
+    constexpr int CH = HC / 8;              // 16-byte chunks of a row
+    static_assert((size_t)BM * LD <= (size_t)S * STAGE, "the tile's outputs do not fit the stages");
+    const int half_n = n / 2;
+    __syncthreads();                        // everyone has read its last fragments
+    const bool upper = (l32 & 16) != 0;
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        // gate rows in lanes 0..15 of a half wave, up rows in lanes 16..31: the two halves swap what
+        // the other needs, the lower one finishing the even tokens and the upper one the odd ones
+        bf16_t* dst = lds + (size_t)(wm0 + 32 * j + 4 * g + (upper ? 1 : 0)) * LD + (wn0 + 32 * i) / 2 + (l32 & 15);
+#pragma unroll
+        for (int e = 0; e < 16; e += 2) {
+          const float mine = upper ? acc[i][j][e + 1] : acc[i][j][e];
+          const float give = upper ? acc[i][j][e] : acc[i][j][e + 1];
+          const float got = __shfl_xor(give, 16);
+          const float gate = upper ? got : mine, up = upper ? mine : got;
+          dst[(size_t)(8 * (e / 4) + (e % 4)) * LD] = f32_to_bf16(silu_f32(gate) * up);
+        }
+      }
+    __syncthreads();
+    const bool wide = (reinterpret_cast<uintptr_t>(c) & 15) == 0 && half_n % 8 == 0;
+    for (int q = tid; q < BM * CH; q += 64 * NWAVES) {
+      const int row = q / CH, ch = q - row * CH;
+      const int mm = m0 + row, col = n0 / 2 + ch * 8;
+      if (mm >= m || col >= half_n) continue;
+      const bf16_t* src = lds + (size_t)row * LD + ch * 8;
+      bf16_t* out = reinterpret_cast<bf16_t*>(c) + (size_t)mm * half_n + col;
+      if (wide && col + 8 <= half_n) {
+        *reinterpret_cast<uint4*>(out) = *reinterpret_cast<const uint4*>(src);
+      } else {
+        for (int u = 0; u < 8 && col + u < half_n; ++u) out[u] = src[u];
+      }
+    }
+    return;
+  }
   float* slab = slabs ? slabs + (size_t)blockIdx.y * m * n : nullptr;      // this slice of K's partial sums
 #pragma unroll
   for (int i = 0; i < TN; ++i)
