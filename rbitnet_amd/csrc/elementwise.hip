@@ -262,6 +262,97 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int n_terms,
   }
 }
 
+// The same with four pairs a thread: 16-byte loads of the projections and the angle tables, 8- and
+// 16-byte stores (bfloat16) instead of 4-byte loads and 2-byte stores.  Needs head sizes that are
+// multiples of 8 and 16-byte aligned rows, which the launcher checks.
+__device__ __forceinline__ float4 sum_terms4(const float* __restrict__ p, int n_terms, size_t stride) {
+  float4 v = *reinterpret_cast<const float4*>(p);
+  for (int t = 1; t < n_terms; ++t) {
+    const float4 e = *reinterpret_cast<const float4*>(p + (size_t)t * stride);
+    v.x += e.x;
+    v.y += e.y;
+    v.z += e.z;
+    v.w += e.w;
+  }
+  return v;
+}
+__device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) {
+  *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+}
+__device__ __forceinline__ void store4(bf16_t* p, float a, float b, float c, float d) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
+}
+
+template <typename TC>
+__global__ void rope_kv_write_vec_kernel(const float* __restrict__ qkv, int n_terms, size_t term_stride,
+                                         const float* __restrict__ cos_t, const float* __restrict__ sin_t, int style,
+                                         TC* __restrict__ q_out, TC* __restrict__ k_pages, TC* __restrict__ v_pages,
+                                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
+                                         const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
+                                         int n_kv, int head_dim) {
+  const int t = blockIdx.x;
+  const int pos = tok_pos[t];
+  const int half = head_dim / 2;
+  const int quads = half / 4;
+  const int row_width = (n_heads + 2 * n_kv) * head_dim;
+  const float* src = qkv + (size_t)t * row_width;
+  const float* cr = cos_t ? cos_t + (size_t)pos * half : nullptr;
+  const float* sr = sin_t ? sin_t + (size_t)pos * half : nullptr;
+  size_t page_base = 0;
+  if (k_pages) {
+    const int page = block_table[(size_t)tok_seq[t] * bt_stride + pos / RB_PAGE];
+    page_base = ((size_t)page * n_kv) * RB_PAGE * head_dim + (size_t)(pos % RB_PAGE) * head_dim;
+  }
+  const int first = q_out ? 0 : n_heads * quads;      // without q_out only k is rotated
+  for (int idx = first + threadIdx.x; idx < (n_heads + n_kv) * quads; idx += blockDim.x) {
+    const int h = idx / quads;
+    const int i = 4 * (idx - h * quads);
+    if (h >= n_heads && !k_pages) break;
+    TC* dst = h < n_heads ? q_out + ((size_t)t * n_heads + h) * head_dim
+                          : k_pages + page_base + (size_t)(h - n_heads) * RB_PAGE * head_dim;
+    float4 c = make_float4(1.f, 1.f, 1.f, 1.f), sn = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (cr) {
+      c = *reinterpret_cast<const float4*>(cr + i);
+      sn = *reinterpret_cast<const float4*>(sr + i);
+    }
+    const float* hp = src + h * head_dim;
+    if (style == 0) {
+      // pairs (2 i, 2 i + 1): eight consecutive values
+      const float4 a = sum_terms4(hp + 2 * i, n_terms, term_stride), b = sum_terms4(hp + 2 * i + 4, n_terms, term_stride);
+      float y[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      if (cr) {
+        rotate_pair(a.x, a.y, c.x, sn.x, y[0], y[1]);
+        rotate_pair(a.z, a.w, c.y, sn.y, y[2], y[3]);
+        rotate_pair(b.x, b.y, c.z, sn.z, y[4], y[5]);
+        rotate_pair(b.z, b.w, c.w, sn.w, y[6], y[7]);
+      }
+      store4(dst + 2 * i, y[0], y[1], y[2], y[3]);
+      store4(dst + 2 * i + 4, y[4], y[5], y[6], y[7]);
+    } else {
+      // pairs (i, i + half): four values of each half
+      const float4 a = sum_terms4(hp + i, n_terms, term_stride), b = sum_terms4(hp + half + i, n_terms, term_stride);
+      float y0[4] = {a.x, a.y, a.z, a.w}, y1[4] = {b.x, b.y, b.z, b.w};
+      if (cr) {
+        rotate_pair(a.x, b.x, c.x, sn.x, y0[0], y1[0]);
+        rotate_pair(a.y, b.y, c.y, sn.y, y0[1], y1[1]);
+        rotate_pair(a.z, b.z, c.z, sn.z, y0[2], y1[2]);
+        rotate_pair(a.w, b.w, c.w, sn.w, y0[3], y1[3]);
+      }
+      store4(dst + i, y0[0], y0[1], y0[2], y0[3]);
+      store4(dst + half + i, y1[0], y1[1], y1[2], y1[3]);
+    }
+  }
+  if (v_pages) {
+    const float* vsrc = src + (size_t)(n_heads + n_kv) * head_dim;
+    for (int idx = 4 * threadIdx.x; idx < n_kv * head_dim; idx += 4 * blockDim.x) {
+      const int h = idx / head_dim;
+      const int d = idx - h * head_dim;
+      const float4 v = sum_terms4(vsrc + idx, n_terms, term_stride);
+      store4(v_pages + page_base + (size_t)h * RB_PAGE * head_dim + d, v.x, v.y, v.z, v.w);
+    }
+  }
+}
+
 extern "C" int rb_rope_kv_write(const float* qkv, int qkv_terms, long long qkv_term_stride, const float* cos,
                                 const float* sin, int style, void* q_out,
                                 void* k_pages, void* v_pages, int cache_dtype, const int32_t* tok_pos,
@@ -276,7 +367,20 @@ extern "C" int rb_rope_kv_write(const float* qkv, int qkv_terms, long long qkv_t
   RB_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rb_rope_kv_write: k and v pages go together");
   if (n_tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  if (cache_dtype == RB_F32)
+  auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const bool vec = head_dim % 8 == 0 && qkv_term_stride % 4 == 0 && aligned(qkv) && aligned(cos) && aligned(sin) &&
+                   aligned(q_out) && aligned(k_pages) && aligned(v_pages);
+  if (vec && cache_dtype == RB_F32)
+    rope_kv_write_vec_kernel<float><<<n_tokens, 256, 0, s>>>(qkv, qkv_terms, (size_t)qkv_term_stride, cos, sin, style,
+                                                             (float*)q_out, (float*)k_pages, (float*)v_pages, tok_pos,
+                                                             tok_seq, block_table, bt_stride, n_heads, n_kv_heads,
+                                                             head_dim);
+  else if (vec && cache_dtype == RB_BF16)
+    rope_kv_write_vec_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(qkv, qkv_terms, (size_t)qkv_term_stride, cos, sin, style,
+                                                              (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages,
+                                                              tok_pos, tok_seq, block_table, bt_stride, n_heads,
+                                                              n_kv_heads, head_dim);
+  else if (cache_dtype == RB_F32)
     rope_kv_write_kernel<float><<<n_tokens, 256, 0, s>>>(qkv, qkv_terms, (size_t)qkv_term_stride, cos, sin, style, (float*)q_out, (float*)k_pages,
                                                          (float*)v_pages, tok_pos, tok_seq, block_table,
                                                          bt_stride, n_heads, n_kv_heads, head_dim);
