@@ -238,8 +238,10 @@ def _attention_ref(q, k_full, v_full, tok_seq, tok_pos, n_heads, n_kv, scale, wi
 
 @pytest.mark.parametrize("style", [0, 1])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_rope_kv_write(lib, style, dtype):
-    n_heads, n_kv, d = 3, 3, 48
+@pytest.mark.parametrize("d", [48, 20])
+def test_rope_kv_write(lib, style, dtype, d):
+    """Head size 48: the kernel that takes four pairs a thread; 20 (no multiple of 8): one pair a thread."""
+    n_heads, n_kv = 3, 3
     past, q_lens = [0, 70, 5], [3, 2, 60]
     g, bt, tok_seq, tok_pos, total = _paged_setup(past, q_lens, n_kv, d, dtype)
     t = sum(q_lens)
