@@ -116,6 +116,19 @@ int rb_sample_workspace_bytes(int n_rows, int vocab);
 int rb_sample(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,
               int32_t* tokens, void* workspace, void* stream);
 
+// rb_sample for callers that cannot allocate device memory: code under HIP graph capture, tight
+// serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The
+// same kernels and the same result as rb_sample, but the chunk statistics go into device memory
+// that the library holds itself (256 KiB on every GPU it runs on, until the process ends), so no
+// workspace is passed and neither this call nor anything under it allocates or frees.
+// Limit: n_rows * ceil(vocab / 4096) <= rb_sample_static_max_stats() (16384: 512 rows of a
+// 128k vocabulary); more is refused with an error and nothing is launched.  The stream must belong
+// to the current device.  All calls on one GPU share that memory: two calls whose kernels may
+// overlap there (different streams, no dependency between them) race; calls on one stream do not.
+int rb_sample_static_max_stats(void);
+int rb_sample_static(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,
+                     int32_t* tokens, void* stream);
+
 // What the GPU reaches, measured the simplest way: rb_probe_read reads `bytes` bytes (a multiple of
 // 16) once with 16-byte loads from `blocks` workgroups of 256 lanes; rb_probe_mfma runs 4 * iters bfloat16 32x32x16 MFMAs in each of `waves`
 // waves (a multiple of 4).  `sink` is one float of device memory that is practically never written.

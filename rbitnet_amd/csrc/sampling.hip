@@ -10,6 +10,8 @@
 // of summation (chunks, segments) cannot move the chosen index.
 #include <math.h>
 
+#include <mutex>
+
 #include "api.h"
 #include "common.h"
 
@@ -204,6 +206,59 @@ extern "C" int rb_sample(const float* logits, int n_rows, int vocab, const float
   ChunkStat* stats = (ChunkStat*)workspace;
   sample_chunk_kernel<<<dim3(n_chunks, n_rows), SAMPLE_THREADS, 0, s>>>(logits, vocab, temperature, stats, n_chunks);
   sample_pick_kernel<<<n_rows, SAMPLE_THREADS, 0, s>>>(logits, vocab, temperature, u, stats, n_chunks, tokens);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- the variant that allocates nothing
+// rb_sample_static is rb_sample with the chunk statistics in device memory that the library
+// itself holds: a file-scope array, one copy on every GPU the library runs on, kept until the
+// process ends.  Nothing in it has to start at zero: the first kernel writes every entry
+// [row, chunk] that the second reads.  The array's name is only a host-side handle; the
+// address that kernels get is asked for once per device with hipGetSymbolAddress and kept.
+#define SAMPLE_STATIC_MAX_STATS 16384      // entries of 16 bytes: 256 KiB per GPU
+#define SAMPLE_STATIC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[SAMPLE_STATIC_MAX_STATS * sizeof(ChunkStat)];
+static void* g_scratch_ptr[SAMPLE_STATIC_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+static int scratch_of_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  RB_REQUIRE(e == hipSuccess, "rb_sample_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  RB_REQUIRE(dev >= 0 && dev < SAMPLE_STATIC_MAX_DEVICES, "rb_sample_static: device %d beyond the %d this library keeps scratch for",
+             dev, SAMPLE_STATIC_MAX_DEVICES);
+  std::lock_guard<std::mutex> guard(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    RB_REQUIRE(e == hipSuccess && p != nullptr, "rb_sample_static: hipGetSymbolAddress failed on device %d: %s", dev,
+               hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int rb_sample_static_max_stats(void) { return SAMPLE_STATIC_MAX_STATS; }
+
+extern "C" int rb_sample_static(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,
+                                int32_t* tokens, void* stream) {
+  RB_REQUIRE(n_rows >= 0 && vocab > 0, "rb_sample_static: bad sizes %d x %d", n_rows, vocab);
+  RB_REQUIRE(temperature == nullptr || u != nullptr, "rb_sample_static: temperature given without uniform numbers");
+  if (n_rows == 0) return 0;
+  const long long n_chunks = ((long long)vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+  RB_REQUIRE(n_chunks <= SAMPLE_MAX_CHUNKS && n_rows <= 65535 && (long long)n_rows * n_chunks <= SAMPLE_STATIC_MAX_STATS,
+             "rb_sample_static: %d rows of %d logits need %lld chunk entries, the built-in scratch holds %d "
+             "(use rb_sample with a workspace)",
+             n_rows, vocab, (long long)n_rows * n_chunks, SAMPLE_STATIC_MAX_STATS);
+  void* ptr = nullptr;
+  if (int rc = scratch_of_current_device(&ptr)) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  ChunkStat* stats = (ChunkStat*)ptr;
+  sample_chunk_kernel<<<dim3((int)n_chunks, n_rows), SAMPLE_THREADS, 0, s>>>(logits, vocab, temperature, stats,
+                                                                             (int)n_chunks);
+  sample_pick_kernel<<<n_rows, SAMPLE_THREADS, 0, s>>>(logits, vocab, temperature, u, stats, (int)n_chunks, tokens);
   RB_LAUNCH_CHECK();
   return 0;
 }
