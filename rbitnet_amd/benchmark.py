@@ -10,7 +10,9 @@ first, so the timed steps run at contexts from 512 upwards (the reference publis
 numbers, so `vs_baseline` is null).  One JSON line is printed.
 
   value               decoded tokens per second at the default batch (8)
-  prefill             one prompt of 2,048 tokens: tokens/s, ms, fraction of the bf16 peak
+  prefill             one prompt of 2,048 tokens: tokens/s, ms (the median of 5 runs after one
+                      that warms up; min_ms beside it), fraction of the bf16 peak
+  config.seq_len      the context the timed steps reach (prompt + warmup + steps + 1)
   roofline            bytes a decode step must read (weights once + live cache) / time
   points              decode tokens/s at batch 1 and 64
 """
@@ -46,6 +48,7 @@ MODELS = {"llama3_8b": ("Llama-3-8B shape", LLAMA3_8B), "llama2_7b": ("Llama-2-7
 PROMPT_LEN = 512
 NEW_TOKENS = 256
 PREFILL_TOKENS = 2048
+PREFILL_RUNS = 5
 
 
 def _sync():
@@ -188,7 +191,7 @@ def main(argv=None) -> int:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic: random N(0,0.02) weights, seeded uniform token ids",
         "config": {
-            "model": model_name, "global_batch": args.batch, "seq_len": longest + NEW_TOKENS,
+            "model": model_name, "global_batch": args.batch, "seq_len": longest + args.warmup + args.steps + 1,
             "prompt_len": args.prompt_len if "," in args.prompt_len else longest, "parallelism": "single GPU", "layers": layers, "layers_full": full_layers,
             "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": hk, "head_dim": d,
             "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
@@ -205,7 +208,7 @@ def main(argv=None) -> int:
         rng = np.random.default_rng(1)
         prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=PREFILL_TOKENS)]
         times = []
-        for i in range(4):
+        for i in range(PREFILL_RUNS + 1):
             slot = engine.alloc_slot()
             _sync()
             t0 = time.perf_counter()
@@ -213,12 +216,13 @@ def main(argv=None) -> int:
             _sync()
             times.append(time.perf_counter() - t0)
             engine.free_slot(slot)
-        pt = min(times[1:])
+        pt = sorted(times[1:])[len(times[1:]) // 2]           # the median; the first run warms up
         layer_flops, head_flops = matmul_flops_per_token(cfg)
         attn_flops = 4.0 * cfg["num_attention_heads"] * d * layers * (PREFILL_TOKENS * (PREFILL_TOKENS + 1) / 2.0)
         flops = layer_flops * PREFILL_TOKENS + head_flops * 1 + attn_flops
         out["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
-                          "frac": round(flops / pt / PEAK_FLOPS[args.dtype], 4)}
+                          "frac": round(flops / pt / PEAK_FLOPS[args.dtype], 4), "runs": PREFILL_RUNS,
+                          "min_ms": round(min(times[1:]) * 1e3, 3)}
         points = {}
         for b in (1, 64):                 # the same prompts and number of steps as the headline batch
             dtb, _ = decode_run(engine, b, args.steps, args.warmup, seed=b, prompt_len=prompt_len)

@@ -36,7 +36,10 @@ class LayerCacheView:
 
 
 class KvGroup:
-    def __init__(self, request: CacheRequest, layers: List[int], n_pages: int, dtype, device):
+    """Keys and values per token in pages; a window gives pages back as a sequence moves on."""
+    kind = "kv"
+
+    def __init__(self, request: CacheRequest, layers: List[int], n_pages: int, n_slots: int, dtype, device):
         self.request = request
         self.layers = list(layers)
         self.index = {l: i for i, l in enumerate(self.layers)}
@@ -45,20 +48,76 @@ class KvGroup:
         self.k = torch.empty(shape, dtype=dtype, device=device)
         self.v = torch.empty(shape, dtype=dtype, device=device)
 
+    @staticmethod
+    def bytes_per_token(request: CacheRequest, n_layers: int, dtype: torch.dtype) -> int:
+        return 2 * n_layers * request.heads * request.head_dim * torch.empty((), dtype=dtype).element_size()
+
+    def open(self, slot: int) -> None:
+        self.table.open(slot)
+
+    def close(self, slot: int) -> None:
+        self.table.close(slot)
+
+    def pages_missing(self, slot: int, n_tokens: int) -> int:
+        return max(0, pages_for(n_tokens) - len(self.table.pages(slot)))
+
+    def fill_view(self, view: "LayerCacheView", i: int, block_tables: Dict[int, torch.Tensor]) -> None:
+        view.k_pages, view.v_pages = self.k[i], self.v[i]
+        view.block_table = block_tables[id(self)]
+
     def bytes(self) -> int:
         return 2 * self.k.numel() * self.k.element_size()
 
 
 class StateGroup:
-    def __init__(self, request: CacheRequest, layers: List[int], n_slots: int, device):
+    """A fixed number of values per sequence, set to their initial value when a slot is handed out."""
+    kind = "state"
+
+    def __init__(self, request: CacheRequest, layers: List[int], n_pages: int, n_slots: int, dtype, device):
         self.request = request
         self.layers = list(layers)
         self.index = {l: i for i, l in enumerate(self.layers)}
         shape = (len(self.layers), n_slots) + tuple(request.state_shape)
         self.data = torch.full(shape, request.state_init, dtype=request.state_dtype, device=device)
 
-    def reset(self, slot: int) -> None:
+    @staticmethod
+    def bytes_per_token(request: CacheRequest, n_layers: int, dtype: torch.dtype) -> int:
+        return 0
+
+    def open(self, slot: int) -> None:
         self.data[:, slot] = self.request.state_init
+
+    def close(self, slot: int) -> None:
+        pass
+
+    def fill_view(self, view: "LayerCacheView", i: int, block_tables: Dict[int, torch.Tensor]) -> None:
+        view.state = self.data[i]
+
+    def bytes(self) -> int:
+        return self.data.numel() * self.data.element_size()
+
+
+# kind of a CacheRequest -> the class that stores it.  A group class has: kind,
+# __init__(request, layers, n_pages, n_slots, dtype, device), open(slot), close(slot),
+# fill_view(view, index in the group, block tables of the step), bytes() and the static
+# bytes_per_token(request, n_layers, dtype); one that grows with the sequence in pages keeps a
+# PageTable as `table`, as KvGroup does, and is then counted when pages are reserved.
+_GROUP_KINDS: Dict[str, type] = {"kv": KvGroup, "state": StateGroup}
+
+
+def register_cache_kind(kind: str, group_class: type) -> None:
+    _GROUP_KINDS[kind] = group_class
+
+
+def bytes_per_token(requests: Sequence[Optional[CacheRequest]], dtype: torch.dtype) -> int:
+    """Bytes that one more token of one sequence adds over all layers."""
+    counts: Dict[Tuple, int] = {}
+    reqs: Dict[Tuple, CacheRequest] = {}
+    for r in requests:
+        if r is not None and r.kind in _GROUP_KINDS:
+            counts[r.key()] = counts.get(r.key(), 0) + 1
+            reqs[r.key()] = r
+    return sum(_GROUP_KINDS[reqs[k].kind].bytes_per_token(reqs[k], n, dtype) for k, n in counts.items())
 
 
 class Cache:
@@ -76,51 +135,52 @@ class Cache:
         self.device = device
         self.slots = FreeList(self.n_slots, "slot")
         self.lens: Dict[int, int] = {}
-        self.kv_groups: List[KvGroup] = []
-        self.state_groups: List[StateGroup] = []
-        self.layer_kv: Dict[int, Tuple[KvGroup, int]] = {}
-        self.layer_state: Dict[int, Tuple[StateGroup, int]] = {}
+        self.groups: List = []
+        self.layer_groups: Dict[int, List[Tuple[object, int]]] = {}
         by_key: Dict[Tuple, List[int]] = {}
         reqs: Dict[Tuple, CacheRequest] = {}
         for l, r in enumerate(requests):
             if r is None:
                 continue
-            if r.kind not in ("kv", "state"):
-                raise CacheError(f"layer {l} asks for an unknown kind of cache {r.kind!r}")
+            if r.kind not in _GROUP_KINDS:
+                raise CacheError(f"layer {l} asks for an unknown kind of cache {r.kind!r} "
+                                 f"(known: {', '.join(sorted(_GROUP_KINDS))})")
             by_key.setdefault(r.key(), []).append(l)
             reqs[r.key()] = r
         for key, layers in by_key.items():
             r = reqs[key]
-            if r.kind == "kv":
-                g = KvGroup(r, layers, self.n_pages, dtype, device)
-                self.kv_groups.append(g)
-                for l in layers:
-                    self.layer_kv[l] = (g, g.index[l])
-            else:
-                s = StateGroup(r, layers, self.n_slots, device)
-                self.state_groups.append(s)
-                for l in layers:
-                    self.layer_state[l] = (s, s.index[l])
+            g = _GROUP_KINDS[r.kind](r, layers, self.n_pages, self.n_slots, dtype, device)
+            self.groups.append(g)
+            for l in layers:
+                self.layer_groups.setdefault(l, []).append((g, g.index[l]))
         for l, j in (readers or {}).items():
-            if j not in self.layer_kv:
+            theirs = [(g, i) for g, i in self.layer_groups.get(j, []) if g.kind == "kv"]
+            if not theirs:
                 raise CacheError(f"layer {l} reads the cache of layer {j}, which keeps none")
-            self.layer_kv[l] = self.layer_kv[j]
+            self.layer_groups.setdefault(l, []).extend(theirs)
+
+    @property
+    def kv_groups(self) -> List:
+        """The groups that grow with their sequences in pages."""
+        return [g for g in self.groups if hasattr(g, "table")]
+
+    @property
+    def state_groups(self) -> List:
+        return [g for g in self.groups if g.kind == "state"]
 
     # ------------------------------------------------------------------ slots
     def alloc_slot(self) -> int:
         slot = self.slots.take()
         self.lens[slot] = 0
-        for g in self.kv_groups:
-            g.table.open(slot)
-        for s in self.state_groups:
-            s.reset(slot)
+        for g in self.groups:
+            g.open(slot)
         return slot
 
     def free_slot(self, slot: int) -> None:
         self.slots.give_back(slot)
         del self.lens[slot]
-        for g in self.kv_groups:
-            g.table.close(slot)
+        for g in self.groups:
+            g.close(slot)
 
     def length(self, slot: int) -> int:
         if slot not in self.lens:
@@ -131,6 +191,26 @@ class Cache:
     def live_slots(self) -> List[int]:
         return self.slots.held()
 
+    # ------------------------------------------------------------------ room, in tokens
+    def token_capacity(self) -> int:
+        """The most tokens all live sequences can hold together, each counted with
+        `tokens_needed` of its length."""
+        return min((g.table.pool.n * PAGE_SIZE for g in self.kv_groups), default=1 << 40)
+
+    @staticmethod
+    def tokens_needed(n_tokens: int) -> int:
+        """What a sequence of n tokens takes of the capacity: whole pages."""
+        return pages_for(n_tokens) * PAGE_SIZE
+
+    def can_grow(self, slot: int, by: int = 1) -> bool:
+        """Whether the sequence can hold `by` more tokens: in the pages it has, or in free ones."""
+        n = self.length(slot) + by
+        return all(g.pages_missing(slot, n) <= g.table.pool.n_free for g in self.kv_groups)
+
+    @staticmethod
+    def pages_per_sequence(n_tokens: int) -> int:
+        return pages_for(n_tokens)
+
     # ------------------------------------------------------------------ steps
     def reserve(self, slots: Sequence[int], q_lens: Sequence[int]) -> None:
         """Pages for the tokens a step is about to write.  All or nothing."""
@@ -139,7 +219,7 @@ class Cache:
         for slot in slots:
             self.length(slot)
         for g in self.kv_groups:
-            need = sum(max(0, pages_for(self.lens[s] + q) - len(g.table.pages(s))) for s, q in zip(slots, q_lens))
+            need = sum(g.pages_missing(s, self.lens[s] + q) for s, q in zip(slots, q_lens))
             if need > g.table.pool.n_free:
                 raise CacheError(
                     f"cache full: the step needs {need} more pages of {PAGE_SIZE} tokens, "
@@ -155,20 +235,18 @@ class Cache:
             for g in self.kv_groups:
                 g.table.release_behind(s, self.lens[s])
 
-    def block_table(self, group: KvGroup, slots: Sequence[int], width: Optional[int] = None) -> List[List[int]]:
-        rows = [group.table.pages(s) for s in slots]
-        w = width or max(1, max(len(r) for r in rows))
-        return [[(p if p >= 0 else 0) for p in r] + [0] * (w - len(r)) for r in rows]
+    def group_keys(self) -> List[int]:
+        return [id(g) for g in self.kv_groups]
+
+    def block_tables(self, slots: Sequence[int]) -> Dict[int, List[List[int]]]:
+        """Per paged group, per sequence of the step, its pages (a page given back behind a
+        window is never read; 0 stands in for it)."""
+        return {id(g): [[(p if p >= 0 else 0) for p in g.table.pages(s)] for s in slots] for g in self.kv_groups}
 
     def view(self, layer: int, block_tables: Dict[int, torch.Tensor]) -> LayerCacheView:
         v = LayerCacheView()
-        if layer in self.layer_kv:
-            g, i = self.layer_kv[layer]
-            v.k_pages, v.v_pages = g.k[i], g.v[i]
-            v.block_table = block_tables[id(g)]
-        if layer in self.layer_state:
-            s, i = self.layer_state[layer]
-            v.state = s.data[i]
+        for g, i in self.layer_groups.get(layer, []):
+            g.fill_view(v, i, block_tables)
         return v
 
     def check(self) -> None:
@@ -181,5 +259,4 @@ class Cache:
                 raise CacheError("a page table exists for a slot that is not in use, or is missing")
 
     def bytes(self) -> int:
-        return sum(g.bytes() for g in self.kv_groups) + sum(
-            s.data.numel() * s.data.element_size() for s in self.state_groups)
+        return sum(g.bytes() for g in self.groups)

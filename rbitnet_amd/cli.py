@@ -45,23 +45,38 @@ def _ids(text: str) -> List[int]:
         raise ConfigError(f"token ids must be integers separated by commas, found {text!r}") from None
 
 
-def _engine(args, max_tokens_hint: int):
+def _cache_need(prompt_lens: List[int], max_tokens: int, max_batch: int, limit: int):
+    """What the request asks of the cache: the longest sequence it can come to, and the most
+    tokens that `max_batch` prompts in a row can come to hold together (each rounded up to the
+    cache's unit of 64 tokens)."""
+    most = [min(n + max_tokens, limit) for n in prompt_lens]
+    rounded = [(n + 63) // 64 * 64 for n in most]
+    together = max(sum(rounded[i:i + max_batch]) for i in range(0, max(1, len(rounded) - max_batch + 1)))
+    return max(most), together
+
+
+def _engine(args, prompt_lens: List[int], max_tokens: int):
+    from .config import load_config
     from .engine import Engine
     model = args.model or os.environ.get("RBITNET_MODEL")
     if os.environ.get("RBITNET_MODEL") and not args.model:
         _no_parent_components(model)
     toy = _truthy("RBITNET_TOY") or getattr(args, "random", False)
-    kw = dict(dtype=args.dtype, max_batch=args.max_batch, max_seq_len=args.max_seq_len)
+    config = (getattr(args, "config", None) or model) if toy else model
+    if not config:
+        raise ConfigError("random weights need --config (a config.json or a folder holding one)" if toy else
+                          "model not loaded; pass --model DIR or set RBITNET_MODEL (or RBITNET_TOY=1 with --config)")
+    # the cache is made for this request, not for the longest context the configuration allows
+    _, spec = load_config(config)
+    limit = min(args.max_seq_len or spec.max_positions, spec.max_positions)
+    longest, together = _cache_need(prompt_lens, max_tokens, args.max_batch, limit)
+    kw = dict(dtype=args.dtype, max_batch=args.max_batch, max_seq_len=args.max_seq_len or longest,
+              max_tokens=together)
     if toy:
-        config = getattr(args, "config", None) or model
-        if not config:
-            raise ConfigError("random weights need --config (a config.json or a folder holding one)")
         seed = args.weight_seed if args.weight_seed is not None else int(os.environ.get("RBITNET_TOY_SEED", "42"))
         cfg_path = os.path.join(config, "config.json") if os.path.isdir(config) else config
         with open(cfg_path) as f:
             return Engine.random(json.load(f), seed=seed, **kw)
-    if not model:
-        raise ConfigError("model not loaded; pass --model DIR or set RBITNET_MODEL (or RBITNET_TOY=1 with --config)")
     return Engine.load_path(model, **kw)
 
 
@@ -79,7 +94,7 @@ def cmd_generate(args) -> int:
                 prompts.append(json.loads(line) if line.startswith("[") else _ids(line))
     if not prompts:
         raise ConfigError("no prompt given (--prompt-ids or --prompt-file)")
-    engine = _engine(args, args.max_tokens)
+    engine = _engine(args, [max(1, len(p)) for p in prompts], args.max_tokens)
     stop = _ids(args.stop_token_ids) if args.stop_token_ids else None
     results = engine.generate(prompts, max_tokens=args.max_tokens, temperature=args.temperature, seed=args.seed,
                               stop_token_ids=stop)

@@ -16,14 +16,21 @@ Keys are the ones a Llama config.json holds (hidden_size, num_hidden_layers,
 ...); the GGUF spellings the reference reads (llama.embedding_length, ...) are
 accepted as alternates.  Not in the reference and accepted here: `head_dim`,
 `rope_scaling` (llama3 rule), `tie_word_embeddings`, `eos_token_id`,
-`bos_token_id`, and `rope_style` ("interleaved" pairs (2i, 2i+1) as the
-reference's rope_inplace does, model.rs:122-136; "half" pairs (i, i + D/2)).
+`bos_token_id`, and `rope_style`: which two numbers of a head the rotation pairs.
+"interleaved" pairs (2i, 2i+1), as the reference's rope_inplace does
+(model.rs:122-136): that fits weight files whose q and k rows were permuted for it
+when they were exported, which the GGUF files that the reference reads are.  "half"
+pairs (i, i + D/2): that fits weights stored under the names of a config.json's own
+folder (`model.layers.N.self_attn.q_proj.weight`), which are not permuted.  Without
+the key the tensor names decide (`with_tensor_names`): GGUF spellings (`blk.N.attn_q`)
+give "interleaved", everything else, and a model without a weight file, "half".
 """
 from __future__ import annotations
 
 import json
 import math
 import os
+import dataclasses
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional
 
@@ -146,7 +153,7 @@ class LlamaConfig:
     vocab_size: int
     rope_theta: float = 10000.0
     rope_scaling: Optional[RopeScaling] = None
-    rope_style: str = "interleaved"
+    rope_style: Optional[str] = None      # None: not said; `effective_rope_style` decides
     rms_norm_eps: float = 1e-5
     max_position_embeddings: int = 2048
     tie_word_embeddings: bool = False
@@ -203,8 +210,8 @@ class LlamaConfig:
         for key in ("attention_bias", "mlp_bias"):
             if d.get(key):
                 raise ConfigError(f"{key}=true is not supported: the Llama dense decoder has no biases")
-        style = d.get("rope_style", "interleaved")
-        if style not in ("interleaved", "half"):
+        style = d.get("rope_style")
+        if style is not None and style not in ("interleaved", "half"):
             raise ConfigError(f"unsupported rope_style {style!r} (supported: 'interleaved', 'half')")
 
         eos = d.get("eos_token_id")
@@ -247,11 +254,12 @@ class LlamaConfig:
             "hidden_act": "silu",
             "rope_theta": self.rope_theta,
             "rope_scaling": self.rope_scaling.as_dict() if self.rope_scaling else None,
-            "rope_style": self.rope_style,
             "rms_norm_eps": self.rms_norm_eps,
             "max_position_embeddings": self.max_position_embeddings,
             "tie_word_embeddings": self.tie_word_embeddings,
         }
+        if self.rope_style is not None:
+            out["rope_style"] = self.rope_style
         if self.eos_token_ids:
             out["eos_token_id"] = self.eos_token_ids if len(self.eos_token_ids) > 1 else self.eos_token_ids[0]
         if self.bos_token_id is not None:
@@ -259,6 +267,19 @@ class LlamaConfig:
         if self.torch_dtype:
             out["torch_dtype"] = self.torch_dtype
         return out
+
+    # ------------------------------------------------------------------ pairing of the rotation
+    def with_tensor_names(self, names) -> "LlamaConfig":
+        """The configuration for a weight file that holds tensors of these names: where
+        config.json does not say how the rotation pairs a head's numbers, files with the GGUF
+        spellings (exported with q and k rows permuted for adjacent pairs) get "interleaved"."""
+        if self.rope_style is None and any(n.startswith("blk.") or n.startswith("token_embd") for n in names):
+            return dataclasses.replace(self, rope_style="interleaved")
+        return self
+
+    @property
+    def effective_rope_style(self) -> str:
+        return self.rope_style or "half"
 
     # ------------------------------------------------------------------ the spec
     def to_spec(self) -> ModelSpec:
@@ -269,7 +290,7 @@ class LlamaConfig:
             "head_dim": self.head_dim,
             "theta": self.rope_theta,
             "scaling": self.rope_scaling.as_dict() if self.rope_scaling else None,
-            "style": self.rope_style,
+            "style": self.effective_rope_style,
             "max_positions": self.max_position_embeddings,
         })
         norm = PartSpec("rmsnorm", {"size": self.hidden_size, "eps": self.rms_norm_eps})
@@ -305,6 +326,8 @@ class LlamaConfig:
             head_name=None if self.tie_word_embeddings else "lm_head.weight",
             stop_token_ids=list(self.eos_token_ids),
             bos_token_id=self.bos_token_id,
+            # an output matrix stored beside tied embeddings is not read
+            optional_tensors=["lm_head.weight"] if self.tie_word_embeddings else [],
         )
 
     # the names a GGUF export of the same model uses (model.rs:146-179), accepted

@@ -6,13 +6,14 @@ keys whatever `general.architecture` says (gguf/bitnet_meta.rs:27-28) and uses
 the name only as a label (gguf/parse.rs:222-234).
 
 A configuration class has: `from_dict(dict)`, `to_dict()`, `to_spec()` and
-optionally `tensor_aliases(name) -> [alternate names]`.
+optionally `tensor_aliases(name) -> [alternate names]` and `with_tensor_names(names)
+-> configuration` (what the names in a weight file decide where config.json is silent).
 """
 from __future__ import annotations
 
 import json
 import os
-from typing import Any, Dict, Tuple
+from typing import Any, Dict, Iterable, Optional, Tuple
 
 from ..errors import ConfigError
 from .llama import LlamaConfig
@@ -49,9 +50,9 @@ def architecture_of(config: Dict[str, Any]) -> str:
     raise ConfigError("config.json names no architecture (key 'architectures')")
 
 
-def load_config(path_or_dict: Any) -> Tuple[Any, ModelSpec]:
+def load_config(path_or_dict: Any, tensor_names: Optional[Iterable[str]] = None) -> Tuple[Any, ModelSpec]:
     """config.json (a folder, a file or an already parsed dict) -> (typed
-    configuration, spec)."""
+    configuration, spec).  tensor_names: the names in the weight file that goes with it."""
     if isinstance(path_or_dict, dict):
         raw = path_or_dict
     else:
@@ -69,6 +70,8 @@ def load_config(path_or_dict: Any) -> Tuple[Any, ModelSpec]:
             raise ConfigError(f"{path} does not hold a JSON object")
     cls = config_class_for(architecture_of(raw))
     cfg = cls.from_dict(raw)
+    if tensor_names is not None and hasattr(cfg, "with_tensor_names"):
+        cfg = cfg.with_tensor_names(list(tensor_names))
     return cfg, cfg.to_spec()
 
 

@@ -58,6 +58,8 @@ class ModelSpec:
     schedule: List[int] = field(default_factory=list)
     stop_token_ids: List[int] = field(default_factory=list)
     bos_token_id: Optional[int] = None
+    # tensors that a weight file may hold without the model reading them
+    optional_tensors: List[str] = field(default_factory=list)
 
     def __post_init__(self) -> None:
         if not self.schedule:

@@ -129,24 +129,22 @@ int rb_sample_static_max_stats(void);
 int rb_sample_static(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,
                      int32_t* tokens, void* stream);
 
+// Load-time helpers (weights_init.hip).
+// rb_fill_normal: out[i] = mean + std * z_i for i < n, z_i the standard normal number that (key, i)
+// fixes; the same bits as weights/random_init.py draws on the host.
+int rb_fill_normal(void* out, int dtype, long long n, unsigned long long key, double mean, double std, void* stream);
+// rb_place_rows: row r of src [n_rows, width] goes, cast to dst's dtype, to row
+// row0 + (r / block) * period + r % block of dst [dst_rows, width].  block = n_rows places the rows
+// one after another from row0 (q, k, v in one matrix); block 16, period 32, row0 0 and 16 interleave
+// gate and up rows in blocks of 16.
+int rb_place_rows(const void* src, int src_dtype, void* dst, int dst_dtype, long long n_rows, long long width,
+                  long long dst_rows, long long row0, long long block, long long period, void* stream);
+
 // What the GPU reaches, measured the simplest way: rb_probe_read reads `bytes` bytes (a multiple of
 // 16) once with 16-byte loads from `blocks` workgroups of 256 lanes; rb_probe_mfma runs 4 * iters bfloat16 32x32x16 MFMAs in each of `waves`
 // waves (a multiple of 4).  `sink` is one float of device memory that is practically never written.
 int rb_probe_read(const void* p, long long bytes, int blocks, float* sink, void* stream);
 int rb_probe_mfma(int waves, int iters, float* sink, void* stream);
-
-// ---- experiment hooks: they override the built-in choice of kernel, tile or wave count for
-// measurements and for tests that must reach a kernel the dispatcher would not pick.  The
-// settings are process-wide and are read at every launch; 0 restores the built-in choice.
-void rb_tune(int stages, int rows_per_wave, int waves);         // skinny product
-void rb_tune_resident(int waves, int parts, int tiles);         // skinny product with resident tokens
-void rb_tune_use_resident(int on);                              // 0: never the resident variant, 2: also below 8192 rows
-void rb_tune_use_stream(int on);                                // 0: the skinny product up to 64 tokens
-void rb_tune_tiles(int cfg, int parts);                         // tiled product: tile configuration and K slices
-void rb_tune_prefill_waves(int waves);                          // prefill attention: 4 or 8
-void rb_tune_prefill_paired(int on);                           // prefill attention: 0 = late blocks first only, no pairing of heavy and light workgroups
-void rb_tune_decode_mfma(int mode);                             // decode attention: 1 matrix cores, 2 vector units
-void rb_tune_decode_waves(int waves);                           // matrix-core decode attention: 4 or 8
 
 #ifdef __cplusplus
 }

@@ -18,6 +18,7 @@
 #include <math.h>
 
 #include "api.h"
+#include "tune.h"
 #include "mfma.h"
 
 #define LOG2E 1.4426950408889634f

@@ -6,6 +6,7 @@
 //    where the tiles alone are too few to fill the GPU (gemm_tiled.hip); 17..64 tokens with a
 //    K that is no multiple of 64: the skinny kernel.
 #include "api.h"
+#include "tune.h"
 #include "gemm_internal.h"
 
 static int g_use_resident = 1, g_use_tiled_small = 1;

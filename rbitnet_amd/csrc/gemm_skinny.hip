@@ -20,6 +20,7 @@
 //
 // Reference loop: y[o] = sum_i W[i + o * n_in] * x[i]  (llama/model.rs:67-91).
 #include "api.h"
+#include "tune.h"
 #include "gemm_internal.h"
 
 struct FoldArgs {

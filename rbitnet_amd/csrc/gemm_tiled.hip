@@ -7,6 +7,7 @@
 //
 // Reference loop: y[o] = sum_i W[i + o * n_in] * x[i]  (llama/model.rs:67-91).
 #include "api.h"
+#include "tune.h"
 #include "gemm_internal.h"
 
 // Adds up the [M, N] slabs of partial sums that the K slices of a product wrote, in slice

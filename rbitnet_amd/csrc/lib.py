@@ -3,9 +3,12 @@ current HIP stream.  There is no fallback: without a GPU and the built library e
 call fails with a KernelError."""
 from __future__ import annotations
 
+import atexit
 import ctypes
+import os
+import sys
 import threading
-from typing import Optional
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
@@ -54,6 +57,49 @@ def _terms(qkv: torch.Tensor, width: int):
     return n, 1, 0
 
 
+class KernelTimes:
+    """Time on the GPU per kernel wrapper, from events recorded around every call: the
+    "wall time per token, then a profiler" checklist of the reference (docs/PROFILING.md:7-11)
+    without leaving the process.  Switched on by RBITNET_KERNEL_TIMES=1 (the decode step is then
+    launched kernel by kernel instead of replayed as a graph, so that every launch can be timed);
+    the table goes to standard error when the process ends, or to whoever calls `report()`."""
+
+    def __init__(self) -> None:
+        self.events: Dict[str, List[Tuple[torch.cuda.Event, torch.cuda.Event]]] = {}
+
+    def wrap(self, name: str, fn):
+        def timed(*args, **kwargs):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            try:
+                return fn(*args, **kwargs)
+            finally:
+                end.record()
+                self.events.setdefault(name, []).append((start, end))
+        return timed
+
+    def totals(self) -> Dict[str, Tuple[int, float]]:
+        """name -> (calls, milliseconds); waits for the GPU."""
+        torch.cuda.synchronize()
+        return {name: (len(pairs), sum(a.elapsed_time(b) for a, b in pairs)) for name, pairs in self.events.items()}
+
+    def reset(self) -> None:
+        self.events.clear()
+
+    def report(self) -> str:
+        totals = self.totals()
+        whole = sum(ms for _, ms in totals.values()) or 1.0
+        lines = [f"{'kernel':32} {'calls':>8} {'total ms':>10} {'mean us':>9} {'share':>6}"]
+        for name, (calls, ms) in sorted(totals.items(), key=lambda kv: -kv[1][1]):
+            lines.append(f"{name:32} {calls:8d} {ms:10.3f} {ms * 1e3 / max(1, calls):9.1f} {ms / whole:6.1%}")
+        return "\n".join(lines)
+
+
+TIMED_OPS = ("embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
+             "gemm_bf16_few", "attention_generic", "attention_prefill_bf16", "attention_decode_bf16",
+             "attention_decode_fused_bf16", "sample")
+
+
 class Kernels:
     """The loaded library.  Methods check operand shapes on the host before a launch, so
     that a kernel never sees sizes other than the ones its grid assumes."""
@@ -86,6 +132,8 @@ class Kernels:
             "rb_attention_decode_fused_bf16": [_P, _I, ctypes.c_longlong, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
                                                _P, _P],
             "rb_sample": [_P, _I, _I, _P, _P, _P, _P, _P],
+            "rb_fill_normal": [_P, _I, ctypes.c_longlong, ctypes.c_ulonglong, ctypes.c_double, ctypes.c_double, _P],
+            "rb_place_rows": [_P, _I, _P, _I] + [ctypes.c_longlong] * 6 + [_P],
             "rb_probe_read": [_P, ctypes.c_longlong, _I, _P, _P],
             "rb_probe_mfma": [_I, _I, _P, _P],
         }
@@ -98,6 +146,13 @@ class Kernels:
         L.rb_sample_workspace_bytes.argtypes = [_I, _I]
         L.rb_sample_workspace_bytes.restype = _I
         self.page_size = int(L.rb_page_size())
+        self.times: Optional[KernelTimes] = None
+        if os.environ.get("RBITNET_KERNEL_TIMES", "") in ("1", "true", "yes"):
+            self.times = KernelTimes()
+            for name in TIMED_OPS:
+                setattr(self, name, self.times.wrap(name, getattr(self, name)))
+            atexit.register(lambda: print(self.times.report(), file=sys.stderr, flush=True))
+        self.n_compute_units = int(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count)
 
     # ------------------------------------------------------------------ helpers
     @staticmethod
@@ -333,6 +388,27 @@ class Kernels:
             raise KernelError("sampling workspace too small")
         self._ok(self._lib.rb_sample(_ptr(logits), n, vocab, _ptr(temperature), _ptr(u), _ptr(tokens),
                                      _ptr(workspace), self._stream()))
+
+    # ------------------------------------------------------------------ load time
+    def fill_normal(self, out: torch.Tensor, key: int, mean: float, std: float) -> None:
+        """out[i] = mean + std * (the standard normal number that (key, i) fixes)."""
+        _check(out, "out")
+        self._ok(self._lib.rb_fill_normal(_ptr(out), dtype_code(out.dtype), out.numel(), int(key) & (2**64 - 1),
+                                          float(mean), float(std), self._stream()))
+
+    def place_rows(self, src: torch.Tensor, dst: torch.Tensor, row0: int = 0, block: Optional[int] = None,
+                   period: Optional[int] = None) -> None:
+        """Row r of src goes, cast to dst's dtype, to row row0 + (r // block) * period + r % block
+        of dst (block: all rows, so that they follow one another from row0)."""
+        _check(src, "src")
+        _check(dst, "dst")
+        if src.dim() != 2 or dst.dim() != 2 or src.shape[1] != dst.shape[1]:
+            raise KernelError(f"place_rows: {tuple(src.shape)} does not fit into {tuple(dst.shape)}")
+        n = src.shape[0]
+        block = max(1, n) if block is None else int(block)
+        period = block if period is None else int(period)
+        self._ok(self._lib.rb_place_rows(_ptr(src), dtype_code(src.dtype), _ptr(dst), dtype_code(dst.dtype), n,
+                                         src.shape[1], dst.shape[0], int(row0), block, period, self._stream()))
 
     # ------------------------------------------------------------------ probes
     def probe_read(self, buf: torch.Tensor, sink: torch.Tensor, blocks: int = 2048) -> None:

@@ -1,0 +1,23 @@
+// Hooks for measurements and for tests that must reach a kernel the dispatcher would not pick.
+// They are no part of the library's interface: nothing on the product path calls them, and
+// only tests and measurement scripts bind them.  The settings are process-wide and are read at
+// every launch; 0 restores the built-in choice.
+#pragma once
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+void rb_tune(int stages, int rows_per_wave, int waves);         // skinny product
+void rb_tune_resident(int waves, int parts, int tiles);         // skinny product with resident tokens
+void rb_tune_use_resident(int on);                              // 0: never the resident variant, 2: also below 8192 rows
+void rb_tune_use_stream(int on);                                // 0: the skinny product up to 64 tokens
+void rb_tune_tiles(int cfg, int parts);                         // tiled product: tile configuration and K slices
+void rb_tune_prefill_waves(int waves);                          // prefill attention: 4 or 8
+void rb_tune_prefill_paired(int on);                           // prefill attention: 0 = late blocks first only, no pairing of heavy and light workgroups
+void rb_tune_decode_mfma(int mode);                             // decode attention: 1 matrix cores, 2 vector units
+void rb_tune_decode_waves(int waves);                           // matrix-core decode attention: 4 or 8
+
+#ifdef __cplusplus
+}
+#endif

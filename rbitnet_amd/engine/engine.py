@@ -12,16 +12,23 @@ the model's or the cache's limit are errors raised before anything is launched.
 """
 from __future__ import annotations
 
+import sys
+from collections import OrderedDict
 from typing import Any, Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
 from ..cache import PAGE_SIZE, Cache, pages_for
+from ..cache.cache import bytes_per_token as cache_bytes_per_token
 from ..config import load_config
-from ..errors import ConfigError, InferenceError
+from ..errors import CacheError, ConfigError, InferenceError
 from ..weights import DEFAULT_SEED, RandomTensors, load_weights
-from .context import StepContext
+from .context import StepBatch, StepContext, split_bucket
 from .model import Model
+
+DEFAULT_MAX_BATCH = 8
+MAX_DECODE_GRAPHS = 24
+CACHE_MEMORY_FRACTION = 0.9       # of the memory that is free after the weights, for a cache nobody sized
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
            torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
@@ -47,8 +54,10 @@ class Engine:
         self.cache = Cache(model.cache_requests(), n_slots=self.max_batch, max_tokens=max_tokens,
                            dtype=self.dtype, device=self.device, readers=model.cache_readers())
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0}
-        self.use_graphs = bool(model.graph_safe)
-        self._graphs: Dict[Tuple[int, int], Any] = {}      # (sequences, split bucket) -> DecodeGraph
+        # per-kernel timers need every launch on its own
+        self.use_graphs = bool(model.graph_safe) and getattr(self.lib, "times", None) is None
+        # (sequences, split bucket) -> DecodeGraph, least recently used first
+        self._graphs: "OrderedDict[Tuple[int, int], Any]" = OrderedDict()
         # float32 [sequences, vocab] of the last `decode_step`, valid until the next one
         self.last_decode_logits: Optional[torch.Tensor] = None
         from ..sampling import Sampler
@@ -56,20 +65,44 @@ class Engine:
 
     # ------------------------------------------------------------------ construction
     @classmethod
-    def _build(cls, config_source: Any, tensors_for, dtype: Any, max_tokens: Optional[int], max_batch: Optional[int],
+    def _build(cls, cfg: Any, spec, tensors_for, dtype: Any, max_tokens: Optional[int], max_batch: Optional[int],
                max_seq_len: Optional[int], device: str, generic_only: bool) -> "Engine":
         from ..csrc.lib import kernels
-        cfg, spec = load_config(config_source)
         lib = kernels()                       # raises when there is no GPU or no built library
         tdtype = parse_dtype(dtype)
-        model = Model(spec, tdtype, device, lib, generic_only=generic_only)
-        model.load(tensors_for(model, cfg))
         seq = min(int(max_seq_len or spec.max_positions), spec.max_positions)
+        model = Model(spec, tdtype, device, lib, generic_only=generic_only, max_seq_len=seq)
+        model.load(tensors_for(model, cfg))
         if max_batch is None:
-            max_batch = 8 if max_tokens is None else max(1, min(pages_for(max_tokens), 1024))
-        if max_tokens is None:
-            max_tokens = max_batch * pages_for(seq) * PAGE_SIZE
+            max_batch = DEFAULT_MAX_BATCH if max_tokens is None else max(1, min(pages_for(max_tokens), 1024))
+        max_tokens = cls._cache_tokens(model, max_tokens, max_batch, seq)
         return cls(cfg, spec, model, max_tokens=max_tokens, max_batch=max_batch, max_seq_len=seq)
+
+    @staticmethod
+    def _cache_tokens(model: Model, max_tokens: Optional[int], max_batch: int, seq: int) -> int:
+        """How many tokens the cache is made for.  Asked for: that many, or an error that says
+        what fits.  Not asked for: every slot at the longest sequence, but no more than the memory
+        that is free once the weights are placed (a message says so)."""
+        per_token = cache_bytes_per_token(model.cache_requests(), model.dtype)
+        fits = 1 << 40
+        if per_token > 0 and model.device.type == "cuda":
+            free, _ = torch.cuda.mem_get_info(model.device)
+            fits = int(free * CACHE_MEMORY_FRACTION) // per_token // PAGE_SIZE * PAGE_SIZE
+        if max_tokens is not None:
+            if pages_for(int(max_tokens)) * PAGE_SIZE > max(fits, PAGE_SIZE):
+                raise CacheError(
+                    f"a cache of max_tokens = {max_tokens} tokens ({per_token} bytes a token) does not fit the "
+                    f"GPU's free memory; {fits} tokens would (lower max_tokens, or max_seq_len and max_batch)")
+            return int(max_tokens)
+        wanted = max_batch * pages_for(seq) * PAGE_SIZE
+        if wanted > fits:
+            print(f"[rbitnet_amd] cache: {max_batch} sequences of {seq} tokens would take "
+                  f"{wanted * per_token / 2**30:.1f} GiB; sized to the {fits} tokens that fit free memory "
+                  f"(give max_tokens or max_seq_len to choose)", file=sys.stderr, flush=True)
+            if fits < PAGE_SIZE:
+                raise CacheError("no memory is left for the cache once the weights are placed")
+            return fits
+        return wanted
 
     @classmethod
     def from_spec(cls, spec, tensors, dtype: Any = "bfloat16", max_tokens: int = 4096, max_batch: int = 8,
@@ -87,12 +120,14 @@ class Engine:
                   generic_only: bool = False) -> "Engine":
         """A model folder (config.json + model.safetensors), as the reference's
         `Engine::load_path` takes a GGUF path (inference.rs:121-133)."""
+        from ..weights.safetensors_io import WeightFolder
+        cfg, spec = load_config(path, tensor_names=WeightFolder(path).names())
+
         def tensors_for(model: Model, cfg):
             aliases = getattr(type(cfg), "tensor_aliases", None)
-            ignored = ["lm_head.weight"] if model.spec.head_name is None else []
-            return load_weights(path, model.expected, aliases=aliases, ignored=ignored)
+            return load_weights(path, model.expected, aliases=aliases, ignored=spec.optional_tensors)
 
-        return cls._build(path, tensors_for, dtype, max_tokens, max_batch, max_seq_len, device, generic_only)
+        return cls._build(cfg, spec, tensors_for, dtype, max_tokens, max_batch, max_seq_len, device, generic_only)
 
     @classmethod
     def random(cls, config: Any, seed: int = DEFAULT_SEED, dtype: Any = "bfloat16", std: float = 0.02,
@@ -100,12 +135,15 @@ class Engine:
                max_seq_len: Optional[int] = None, device: str = "cuda:0", generic_only: bool = False) -> "Engine":
         """Random weights drawn on the GPU from a configuration and a seed, no files: the
         counterpart of the reference's toy mode (RBITNET_TOY / RBITNET_TOY_SEED,
-        inference.rs:24-36)."""
+        inference.rs:24-36).  The same model, bit for bit, as `write_random_model` with the
+        same arguments writes (its stored dtype being this compute dtype)."""
+        cfg, spec = load_config(config)
+
         def tensors_for(model: Model, cfg):
             store = torch.bfloat16 if model.dtype == torch.bfloat16 else torch.float32
             return RandomTensors(model.expected, seed, std, norm_std, store, device)
 
-        return cls._build(config, tensors_for, dtype, max_tokens, max_batch, max_seq_len, device, generic_only)
+        return cls._build(cfg, spec, tensors_for, dtype, max_tokens, max_batch, max_seq_len, device, generic_only)
 
     # ------------------------------------------------------------------ slots
     def alloc_slot(self) -> int:
@@ -161,8 +199,8 @@ class Engine:
             base += len(toks)
         q_lens = [len(t) for t in tokens]
         self.cache.reserve(slots, q_lens)
-        tables = {id(g): self.cache.block_table(g, slots) for g in self.cache.kv_groups}
-        ctx = StepContext(self.device, slots, past, tokens, rows, tables)
+        ctx = StepContext.for_batch(self.device, StepBatch(slots, past, tokens, rows, self.cache.block_tables(slots)),
+                                    n_compute_units=self.lib.n_compute_units)
         logits = self.model.forward(ctx, self.cache, ctx.rows)
         self.cache.commit(slots, q_lens)
         self.stats["steps"] += 1
@@ -188,16 +226,17 @@ class Engine:
             logits = self.step([(s, [t]) for s, t in zip(slots, tokens)], "last")
             self.last_decode_logits = logits
             return self.sampler.sample(logits, temperatures, uniforms)
-        from .context import split_bucket
         from .decode_graph import DecodeGraph
         n = len(slots)
         key = (n, split_bucket(max(self.cache.length(s) for s in slots) + 1))
         if key not in self._graphs:
-            if len(self._graphs) >= 24:
-                self._graphs.pop(next(iter(self._graphs)))
+            if len(self._graphs) >= MAX_DECODE_GRAPHS:
+                self._graphs.popitem(last=False)           # the least recently used
             self._graphs[key] = DecodeGraph(self, n, key[1])
-        out = self._graphs[key].run(slots, tokens, temperatures, uniforms)
-        self.last_decode_logits = self._graphs[key].logits
+        self._graphs.move_to_end(key)
+        graph = self._graphs[key]
+        out = graph.run(slots, tokens, temperatures, uniforms)
+        self.last_decode_logits = graph.logits if graph.first_logits is None else graph.first_logits
         self.stats["steps"] += 1
         self.stats["decode_tokens"] += n
         return out

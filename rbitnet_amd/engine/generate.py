@@ -14,15 +14,15 @@ max_tokens does not feed its last token.
 
 `engine` needs: alloc_slot(), free_slot(slot), step(entries, want) -> logits,
 sampler.sample(logits, temperatures, uniforms) -> tokens, decode_step(slots, tokens,
-temperatures, uniforms) -> tokens, max_batch, max_seq_len,
-cache.n_pages / cache.kv_groups (for admission), spec.stop_token_ids.
+temperatures, uniforms) -> tokens, max_batch, max_seq_len, spec.stop_token_ids and, for
+admission, cache.token_capacity(), cache.tokens_needed(n) and cache.can_grow(slot): the
+loop counts tokens and leaves to the cache how it stores them.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import List, Optional, Sequence
+from typing import Callable, List, Optional, Sequence
 
-from ..cache.pages import pages_for
 from ..errors import InferenceError
 from ..sampling.sampler import uniform
 
@@ -57,17 +57,18 @@ def decide(token: int, emitted: int, max_tokens: int, room_after: int, stop_ids)
 
 
 def plan_batches(prompt_lens: Sequence[int], max_tokens: int, max_batch: int, max_seq_len: int,
-                 page_budget: int) -> List[List[int]]:
-    """Requests in order, cut into batches that fit the slots and the pages: a request
-    counts with the most tokens it can come to hold."""
+                 capacity: int, needed: Callable[[int], int] = lambda n: n) -> List[List[int]]:
+    """Requests in order, cut into batches that fit the slots and the cache: a request counts
+    with the most tokens it can come to hold, `needed(n)` being what n tokens take of the
+    cache's `capacity`."""
     batches: List[List[int]] = []
     cur: List[int] = []
     used = 0
     for i, n in enumerate(prompt_lens):
-        need = pages_for(min(n + max_tokens, max_seq_len))
-        if need > page_budget:
-            need = page_budget            # it will end with "context" when the pages run out
-        if cur and (len(cur) >= max_batch or used + need > page_budget):
+        need = needed(min(n + max_tokens, max_seq_len))
+        if need > capacity:
+            need = capacity               # it will end with "context" when the cache is full
+        if cur and (len(cur) >= max_batch or used + need > capacity):
             batches.append(cur)
             cur, used = [], 0
         cur.append(i)
@@ -96,11 +97,13 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 256, te
         for r in results:
             r.finish_reason = "length"
         return results
-    page_budget = min((g.table.pool.n for g in engine.cache.kv_groups), default=1 << 30)
+    cache = engine.cache
+    capacity = cache.token_capacity()
     for i, p in enumerate(prompts):
-        if pages_for(len(p)) > page_budget:
+        if cache.tokens_needed(len(p)) > capacity:
             raise InferenceError(f"request {i}: prompt of {len(p)} tokens does not fit the cache")
-    batches = plan_batches([len(p) for p in prompts], max_tokens, engine.max_batch, engine.max_seq_len, page_budget)
+    batches = plan_batches([len(p) for p in prompts], max_tokens, engine.max_batch, engine.max_seq_len, capacity,
+                           cache.tokens_needed)
 
     for batch in batches:
         running: List[_Running] = []
@@ -121,8 +124,8 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 256, te
                     if verdict != "stop":
                         r.result.tokens.append(int(tok))
                         r.room -= 1
-                    # a sequence that cannot get another page ends here as well
-                    if verdict is None and not _has_page_for(engine, r.slot):
+                    # a sequence that the cache cannot let grow ends here as well
+                    if verdict is None and not cache.can_grow(r.slot):
                         verdict = "context"
                     if verdict is None:
                         survivors.append(r)
@@ -141,12 +144,3 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 256, te
                 if r.slot >= 0:
                     engine.free_slot(r.slot)
     return results
-
-
-def _has_page_for(engine, slot: int) -> bool:
-    """Whether one more token fits the sequence's pages or a free page is left."""
-    n = engine.cache.length(slot)
-    for g in engine.cache.kv_groups:
-        if pages_for(n + 1) > len(g.table.pages(slot)) and g.table.pool.n_free == 0:
-            return False
-    return True

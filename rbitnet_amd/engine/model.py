@@ -66,7 +66,8 @@ def expected_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:
 class Model:
     takes_gained_rows = True      # the output product takes what the last product left for the final norm
 
-    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device, lib, generic_only: bool = False):
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device, lib, generic_only: bool = False,
+                 max_seq_len: Optional[int] = None):
         if dtype not in (torch.float32, torch.bfloat16):
             raise ConfigError(f"compute dtype must be float32 or bfloat16, not {dtype}")
         self.spec = spec
@@ -80,6 +81,7 @@ class Model:
             env = BuildEnv(hidden_size=spec.hidden_size, dtype=dtype, device=self.device, lib=lib, layer_index=i,
                            shared=shared)
             env.generic_only = generic_only
+            env.max_seq_len = max_seq_len         # tables keyed by position need no more rows than this
             return env
 
         self.blocks = _build_blocks(spec, env_for)
@@ -128,11 +130,21 @@ class Model:
 
     # ------------------------------------------------------------------ weights
     def _place(self, t: torch.Tensor, ts: TensorSpec) -> torch.Tensor:
+        """The tensor on the GPU in the dtype its role asks for; a change of the floating type
+        is done there by the library's own copy kernel."""
         if ts.role == "table":
             return t.to(device=self.device, dtype=torch.int32).contiguous()
-        if ts.role == "gain":
-            return t.to(device=self.device, dtype=torch.float32).contiguous()
-        return t.to(device=self.device, dtype=self.dtype).contiguous()
+        want = torch.float32 if ts.role == "gain" else self.dtype
+        t = t.to(device=self.device).contiguous()
+        if t.dtype == want:
+            return t
+        if t.dtype not in (torch.float32, torch.bfloat16):
+            return t.to(want)
+        out = torch.empty(t.shape, dtype=want, device=self.device)
+        if t.numel():
+            width = t.shape[-1] if t.dim() >= 1 else 1
+            self.lib.place_rows(t.reshape(-1, width), out.view(-1, width))
+        return out
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         """tensors: full name -> tensor (any device, stored dtype).  Each is moved to the

@@ -77,8 +77,13 @@ class Attention(Part):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         # q, k and v rows in one matrix: one product per step instead of three
         if self.cache_from is None:
-            self.w_qkv = torch.cat([tensors[self.names["q"]], tensors[self.names["k"]],
-                                    tensors[self.names["v"]]], dim=0).contiguous()
+            parts = [tensors[self.names[n]] for n in ("q", "k", "v")]
+            self.w_qkv = torch.empty((sum(p.shape[0] for p in parts), self.hidden), dtype=parts[0].dtype,
+                                     device=parts[0].device)
+            row = 0
+            for p in parts:
+                self.env.lib.place_rows(p.contiguous(), self.w_qkv, row0=row)
+                row += p.shape[0]
         else:
             self.w_qkv = tensors[self.names["q"]].contiguous()
         self.w_o = tensors[self.names["o"]].contiguous()

@@ -49,6 +49,8 @@ class BuildEnv:
     # one dictionary for all layers of a model: read-only data (tables) that parts with equal
     # parameters build once and share, keyed by the part
     shared: Dict[Any, Any] = field(default_factory=dict)
+    generic_only: bool = False            # never the matrix-core kernels (tests of the generic ones)
+    max_seq_len: Optional[int] = None     # the longest sequence the engine will run, if it is known
 
 
 @dataclass

@@ -45,7 +45,7 @@ class SwiGLU(Part):
                 self.names["down"]: TensorSpec((self.hidden, self.ff))}
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.w_gate_up = pack_gate_up(tensors[self.names["gate"]], tensors[self.names["up"]], self.fused)
+        self.w_gate_up = pack_gate_up(self.env.lib, tensors[self.names["gate"]], tensors[self.names["up"]], self.fused)
         self.w_down = tensors[self.names["down"]].contiguous()
 
     def forward(self, h, ctx=None, stream: Optional[torch.Tensor] = None, next_norm=None):

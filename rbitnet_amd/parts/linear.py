@@ -12,7 +12,6 @@ between them; otherwise the caller is left with the sum and the rows are normali
 """
 from __future__ import annotations
 
-import os
 from typing import Optional
 
 import torch
@@ -27,14 +26,14 @@ def uses_matrix_cores(dtype: torch.dtype, k: int) -> bool:
     return dtype == torch.bfloat16 and k % 8 == 0
 
 
-# RBITNET_FOLD=0 (measurements only): sums and norms stay kernels of their own
-_FOLD = os.environ.get("RBITNET_FOLD", "1") != "0"
+# False (tests and measurements set it): sums and norms stay kernels of their own
+FOLD_INTO_PRODUCTS = True
 
 
 def _few(lib, x, w: torch.Tensor) -> bool:
     """Whether the kernel for a few tokens, which folds its neighbours in, takes this product."""
     m, k = x.shape
-    return _FOLD and uses_matrix_cores(x.dtype, k) and lib.gemm_bf16_few_ok(m, w.shape[0], k)
+    return FOLD_INTO_PRODUCTS and uses_matrix_cores(x.dtype, k) and lib.gemm_bf16_few_ok(m, w.shape[0], k)
 
 
 def _from_gained(lib, x: GainedRows, w: torch.Tensor, out: torch.Tensor, epilogue: int) -> None:
@@ -98,16 +97,19 @@ def can_fuse_gate(dtype: torch.dtype, k: int, ff: int) -> bool:
     return uses_matrix_cores(dtype, k) and ff % GATE_BLOCK == 0
 
 
-def pack_gate_up(gate: torch.Tensor, up: torch.Tensor, fused: bool) -> torch.Tensor:
+def pack_gate_up(lib, gate: torch.Tensor, up: torch.Tensor, fused: bool) -> torch.Tensor:
     """One matrix for both products.  Plain: gate rows, then up rows.  Fused: blocks of
     16 gate rows followed by the 16 up rows of the same columns, so that one lane of the
     matrix-core tile holds a gate value and its up value."""
     ff, k = gate.shape
-    if not fused:
-        return torch.cat([gate, up], dim=0).contiguous()
-    g = gate.reshape(ff // GATE_BLOCK, GATE_BLOCK, k)
-    u = up.reshape(ff // GATE_BLOCK, GATE_BLOCK, k)
-    return torch.stack([g, u], dim=1).reshape(2 * ff, k).contiguous()
+    out = torch.empty((2 * ff, k), dtype=gate.dtype, device=gate.device)
+    if fused:
+        lib.place_rows(gate.contiguous(), out, row0=0, block=GATE_BLOCK, period=2 * GATE_BLOCK)
+        lib.place_rows(up.contiguous(), out, row0=GATE_BLOCK, block=GATE_BLOCK, period=2 * GATE_BLOCK)
+    else:
+        lib.place_rows(gate.contiguous(), out, row0=0)
+        lib.place_rows(up.contiguous(), out, row0=ff)
+    return out
 
 
 def gated_linear(lib, x, w_packed: torch.Tensor, ff: int, fused: bool) -> torch.Tensor:

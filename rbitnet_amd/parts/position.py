@@ -63,6 +63,8 @@ class Rope(Part):
         if self.style is None:
             raise ConfigError(f"unknown rope style {params.get('style')!r}")
         self.max_positions = int(params["max_positions"])
+        if getattr(env, "max_seq_len", None):
+            self.max_positions = min(self.max_positions, int(env.max_seq_len))
         self.env = env
         inv = rope_inverse_frequencies(self.head_dim, float(params["theta"]), params.get("scaling"))
         self.inv_freq = inv

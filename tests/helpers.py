@@ -15,7 +15,7 @@ TINY_A = {
     "architectures": ["LlamaForCausalLM"], "hidden_size": 64, "num_hidden_layers": 2,
     "num_attention_heads": 4, "num_key_value_heads": 2, "intermediate_size": 172, "vocab_size": 256,
     "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 128,
-    "tie_word_embeddings": False,
+    "tie_word_embeddings": False, "rope_style": "interleaved",      # the reference's pairing; B has none: "half"
 }
 TINY_B = {
     "architectures": ["LlamaForCausalLM"], "hidden_size": 96, "num_hidden_layers": 3,
@@ -79,6 +79,19 @@ def plain_logits(name: str, tokens: tuple) -> torch.Tensor:
     return _plain(name).logits(list(tokens))
 
 
+@lru_cache(maxsize=None)
+def _plain_rounded(name: str):
+    from plain_llama import PlainLlama
+    return PlainLlama.from_folder(model_folder(name), round_bf16=True)
+
+
+@lru_cache(maxsize=None)
+def plain_logits_rounded(name: str, tokens: tuple) -> torch.Tensor:
+    """The plain implementation rounding to bfloat16 where an engine that computes in bfloat16
+    stores values in that type: what such an engine can come close to."""
+    return _plain_rounded(name).logits(list(tokens))
+
+
 def max_err(got: torch.Tensor, want: torch.Tensor) -> float:
     """Largest absolute difference relative to the largest wanted magnitude."""
     want = want.to(torch.float64)
@@ -90,3 +103,30 @@ def max_err(got: torch.Tensor, want: torch.Tensor) -> float:
 # summation order and float32 rounding only; bfloat16 rounds activations to 8 bits of
 # mantissa at each layer boundary
 TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+# The bfloat16 engine against the plain implementation that rounds where the engine stores
+# bfloat16.  The two cannot agree value by value: a difference far below one rounding step before
+# a value is rounded becomes a whole step with the matching probability, so after a few roundings
+# in a row two computations that round at the same places are as far from each other as each is
+# from the exact result.  What they share is the size of that distance: its root mean square over
+# a request's logits is a stable number (the engine's is 0.93 to 1.05 of the plain one's over sixty
+# requests of four models; 0.84 to 1.13 over the 8 x V logits of steps of single tokens), so a
+# systematic error of a thousandth of the largest logit already shows.
+BF16_RMS_RATIO = 1.15          # a step of many tokens
+BF16_RMS_RATIO_FEW = 1.3       # 8 single-token steps (fewer logits, folded norms)
+BF16_MAX_RATIO = 1.5           # the largest error against the plain one's largest
+
+
+def rms_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    """Root mean square difference relative to the largest wanted magnitude."""
+    want = want.to(torch.float64)
+    got = got.detach().to("cpu", torch.float64)
+    return float(((got - want) ** 2).mean().sqrt() / want.abs().max().clamp_min(1e-30))
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor, block: int = 16) -> torch.Tensor:
+    """Blocks of 16 gate rows, each followed by the 16 up rows of the same columns: the layout
+    the gated product's epilogue reads, built here with torch as the oracle of the packing kernel."""
+    ff, k = gate.shape
+    g = gate.reshape(ff // block, block, k)
+    u = up.reshape(ff // block, block, k)
+    return torch.stack([g, u], dim=1).reshape(2 * ff, k).contiguous()

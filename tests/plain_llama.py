@@ -139,7 +139,7 @@ def rope(x: torch.Tensor, pos: int, inv_freq: torch.Tensor, style: str = "interl
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_head: int, n_kv: int,
-              window: int | None = None, first_pos: int = 0) -> torch.Tensor:
+              window: int | None = None, first_pos: int = 0, round_weights=None) -> torch.Tensor:
     """Causal attention of a whole sequence, grouped heads.
 
     q [T, n_head*D], k and v [T, n_kv*D], already rotated.  Query head qh reads
@@ -147,7 +147,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_head: int, n_
     product times 1/sqrt(D), the scale applied after the sum (model.rs:260,
     269-275); keys p <= pos only (model.rs:266); softmax; weighted sum of the
     values (model.rs:278-288); heads are concatenated in head order.
-    Ours: `window` keeps only the keys with pos - p < window.
+    Ours: `window` keeps only the keys with pos - p < window; `round_weights`, a function,
+    is applied to the exponentials exp(s - max) before they weigh the values (their sum is
+    taken before it): the place where an engine that multiplies in reduced precision rounds.
     """
     t_len = q.shape[0]
     d = q.shape[1] // n_head
@@ -161,7 +163,11 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_head: int, n_
             qv = q[pos, qh * d:(qh + 1) * d]
             keys = k[lo:pos + 1, kvh * d:(kvh + 1) * d]
             scores = (keys * qv[None, :]).sum(dim=1) * scale
-            prob = softmax(scores)
+            if round_weights is None:
+                prob = softmax(scores)
+            else:
+                z = torch.exp(scores - scores.max())
+                prob = round_weights(z) / z.sum()
             comb = (prob[:, None] * v[lo:pos + 1, kvh * d:(kvh + 1) * d]).sum(dim=0)
             out[pos, qh * d:(qh + 1) * d] = comb
     return out
@@ -179,8 +185,14 @@ def swiglu(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: to
 class PlainLlama:
     """config.json + tensors by name -> logits of whole sequences."""
 
-    def __init__(self, config: dict, tensors: dict, dtype=torch.float64, device="cpu"):
+    def __init__(self, config: dict, tensors: dict, dtype=torch.float64, device="cpu", round_bf16: bool = False):
+        """round_bf16: round to bfloat16 wherever an engine that computes in bfloat16 stores a
+        value in that type (normalised rows, rotated q and k, v, the weights of the values, the
+        attention output, the gated activation), everything else as before.  The distance of
+        that from the exact logits is what such an engine cannot avoid; its distance from an
+        engine's logits is what the engine adds."""
         c = config
+        self.round_bf16 = round_bf16
         self.dtype = dtype
         self.device = device        # where the sums run; the element-by-element rotation stays on the host
         self.n_embd = int(c["hidden_size"])
@@ -193,19 +205,25 @@ class PlainLlama:
         self.theta = float(c.get("rope_theta", 10000.0))                   # config.rs:94-97
         self.eps = float(c.get("rms_norm_eps", 1e-5))                      # config.rs:99-102
         self.scaling = c.get("rope_scaling")
-        self.style = c.get("rope_style", "interleaved")
+        # without the key: "half", the layout of weights stored under these names (this class
+        # reads `model.layers.N...` names only); the reference's adjacent pairs fit GGUF files,
+        # whose q and k rows were permuted for them when they were exported
+        self.style = c.get("rope_style") or "half"
         self.tied = bool(c.get("tie_word_embeddings", False))
         self.window = c.get("sliding_window")
         self.inv_freq = rope_inv_freq(self.head_dim, self.theta, self.scaling)
         self.w = {k: v.to(device=device, dtype=dtype) for k, v in tensors.items()}
 
     @classmethod
-    def from_folder(cls, folder: str, dtype=torch.float64, device="cpu") -> "PlainLlama":
+    def from_folder(cls, folder: str, dtype=torch.float64, device="cpu", round_bf16: bool = False) -> "PlainLlama":
         from safetensors.torch import load_file
         with open(os.path.join(folder, "config.json")) as f:
             config = json.load(f)
         tensors = load_file(os.path.join(folder, "model.safetensors"))
-        return cls(config, tensors, dtype, device)
+        return cls(config, tensors, dtype, device, round_bf16)
+
+    def _r(self, t: torch.Tensor) -> torch.Tensor:
+        return t.to(torch.bfloat16).to(t.dtype) if self.round_bf16 else t
 
     def layer(self, x: torch.Tensor, il: int) -> torch.Tensor:
         """One block: norm, q/k/v, rotate q and k, attention, output projection
@@ -213,7 +231,7 @@ class PlainLlama:
         p = f"model.layers.{il}."
         w = self.w
         d = self.head_dim
-        h = rmsnorm(x, w[p + "input_layernorm.weight"], self.eps)
+        h = self._r(rmsnorm(x, w[p + "input_layernorm.weight"], self.eps))
         q = linear(h, w[p + "self_attn.q_proj.weight"])
         k = linear(h, w[p + "self_attn.k_proj.weight"])
         v = linear(h, w[p + "self_attn.v_proj.weight"])
@@ -223,10 +241,14 @@ class PlainLlama:
                 q[pos, hh * d:(hh + 1) * d] = rope(q[pos, hh * d:(hh + 1) * d], pos, self.inv_freq, self.style)
             for hh in range(self.n_kv):
                 k[pos, hh * d:(hh + 1) * d] = rope(k[pos, hh * d:(hh + 1) * d], pos, self.inv_freq, self.style)
-        q, k = q.to(x.device), k.to(x.device)
-        a = attention(q, k, v, self.n_head, self.n_kv, self.window)
+        q, k, v = self._r(q.to(x.device)), self._r(k.to(x.device)), self._r(v)
+        a = self._r(attention(q, k, v, self.n_head, self.n_kv, self.window,
+                              round_weights=self._r if self.round_bf16 else None))
         x = x + linear(a, w[p + "self_attn.o_proj.weight"])
-        h2 = rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps)
+        h2 = self._r(rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps))
+        if self.round_bf16:
+            t = self._r(silu(linear(h2, w[p + "mlp.gate_proj.weight"])) * linear(h2, w[p + "mlp.up_proj.weight"]))
+            return x + linear(t, w[p + "mlp.down_proj.weight"])
         x = x + swiglu(h2, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                        w[p + "mlp.down_proj.weight"])
         return x
@@ -240,7 +262,7 @@ class PlainLlama:
     def logits(self, tokens) -> torch.Tensor:
         """Logits [T, V] at every position of one sequence.  model.rs:229-315."""
         x = self.hidden(tokens)
-        xn = rmsnorm(x, self.w["model.norm.weight"], self.eps)
+        xn = self._r(rmsnorm(x, self.w["model.norm.weight"], self.eps))
         head = self.w["model.embed_tokens.weight"] if self.tied else self.w["lm_head.weight"]
         return linear(xn, head)
 

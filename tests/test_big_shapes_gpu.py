@@ -1,10 +1,17 @@
 """The kernels that only wide models select (256 x 256 tiles, the token-resident and the
 panel products, flash attention over many blocks, decode splits) at the widths of Llama-3-8B
-with two layers: the float32 engine against the plain implementation, and the bfloat16
-engine's prompt step, decode steps and a mid-size batch against the float32 engine."""
+with two layers and of Llama-3.1-70B with one: the float32 and the bfloat16 engine against the
+plain implementation, for batches of unequal lengths whose longest request spans five pages of
+the cache, the last tokens one by one, one batch after another in the same slots.  Then the
+bfloat16 engine's drift from the float32 engine over twenty requests."""
+import os
+import sys
+
 import numpy as np
 import pytest
 import torch
+
+sys.path.insert(0, os.path.dirname(__file__))
 
 pytestmark = pytest.mark.gpu
 
@@ -15,6 +22,20 @@ WIDE = {
     "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
                      "original_max_position_embeddings": 1024},
 }
+WIDER = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 8192, "num_hidden_layers": 1,
+    "num_attention_heads": 64, "num_key_value_heads": 8, "intermediate_size": 28672, "vocab_size": 128256,
+    "rope_theta": 500000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 8192,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+}
+TAIL = 3                                   # tokens of each request that are fed one by one
+BATCHES = {"wide": [[300, 130, 65, 1], [66, 20]], "wider": [[200, 70, 1]]}
+
+
+def _requests(kind):
+    rng = np.random.default_rng(11)
+    return [[[int(t) for t in rng.integers(0, 128256, size=n)] for n in lengths] for lengths in BATCHES[kind]]
 
 
 @pytest.fixture(scope="module")
@@ -25,37 +46,95 @@ def folder(tmp_path_factory):
     return rbitnet_amd.write_random_model(path, WIDE, seed=5, std=0.03, norm_std=0.05, dtype=torch.bfloat16)
 
 
+@pytest.fixture(scope="module")
+def wider_folder(tmp_path_factory):
+    import rbitnet_amd
+    path = str(tmp_path_factory.mktemp("wider") / "m")
+    return rbitnet_amd.write_random_model(path, WIDER, seed=6, std=0.02, norm_std=0.05, dtype=torch.bfloat16)
+
+
+def _plain_logits(path, kind):
+    """float64 logits of the plain implementation for every request (its sums run on the GPU
+    for their size), computed once per folder."""
+    from plain_llama import PlainLlama
+    plain = PlainLlama.from_folder(path, device="cuda:0")
+    out = [[plain.logits(r).cpu() for r in batch] for batch in _requests(kind)]
+    del plain
+    torch.cuda.empty_cache()
+    return out
+
+
+@pytest.fixture(scope="module")
+def wide_plain(folder):
+    return _plain_logits(folder, "wide")
+
+
+@pytest.fixture(scope="module")
+def wider_plain(wider_folder):
+    return _plain_logits(wider_folder, "wider")
+
+
 def _rel(a, b):
     return float((a.double() - b.double()).abs().max() / b.double().abs().max())
 
 
-def test_wide_model_float32_against_plain(folder):
-    """The float32 engine at full width (sums over 4,096 and 14,336 terms, a vocabulary of
-    128,256) against the plain implementation in float64, whose sums run on the GPU for their
-    size: a prompt in one step, then tokens one by one."""
-    import os
-    import sys
-    sys.path.insert(0, os.path.dirname(__file__))
+def _batches_against_plain(path, kind, want, dtype, tol):
+    """Each batch: the prompts (all but the last TAIL tokens) in one step, then one token each,
+    requests with fewer tokens ending earlier; the next batch in the same slots, whose pages are
+    filled with NaN in between."""
     import rbitnet_amd
-    from plain_llama import PlainLlama
-    rng = np.random.default_rng(11)
-    tokens = [int(t) for t in rng.integers(0, 128256, size=40)]
-    plain = PlainLlama.from_folder(folder, device="cuda:0")
-    want = plain.logits(tokens).cpu()
-    del plain
+    batches = _requests(kind)
+    n_slots = max(len(b) for b in batches)
+    need = max(sum((len(r) + 63) // 64 * 64 for r in b) for b in batches)
+    eng = rbitnet_amd.Engine.load_path(path, dtype=dtype, max_tokens=need, max_batch=n_slots)
+    for reqs, logits_want in zip(batches, want):
+        for g in eng.cache.kv_groups:
+            g.k.fill_(float("nan"))
+            g.v.fill_(float("nan"))
+        slots = [eng.alloc_slot() for _ in reqs]
+        heads = [max(1, len(r) - TAIL) for r in reqs]
+        got = [[] for _ in reqs]
+        logits = eng.step([(s, r[:h]) for s, r, h in zip(slots, reqs, heads)], "all")
+        off = 0
+        for i, h in enumerate(heads):
+            got[i].append(logits[off:off + h].cpu())
+            off += h
+        for j in range(TAIL):
+            live = [i for i, (r, h) in enumerate(zip(reqs, heads)) if h + j < len(r)]
+            if not live:
+                break
+            logits = eng.step([(slots[i], [reqs[i][heads[i] + j]]) for i in live], "last").cpu()
+            for row, i in enumerate(live):
+                got[i].append(logits[row:row + 1])
+        for s in slots:
+            eng.free_slot(s)
+        for i, (r, w) in enumerate(zip(reqs, logits_want)):
+            g = torch.cat(got[i])
+            assert g.shape == w.shape
+            err = (g.double() - w).abs().amax(dim=1) / w.abs().max()
+            assert float(err.max()) < tol, f"{kind} {dtype}: request of {len(r)} tokens, position {int(err.argmax())}: {float(err.max())}"
+    eng.cache.check()
+    assert eng.cache.slots.n_held == 0
+    del eng
     torch.cuda.empty_cache()
-    eng = rbitnet_amd.Engine.load_path(folder, dtype="float32", max_tokens=64, max_batch=1)
-    slot = eng.alloc_slot()
-    got = [eng.step([(slot, tokens[:34])], "all")]
-    for t in tokens[34:]:
-        got.append(eng.step([(slot, [t])], "last"))
-    eng.free_slot(slot)
-    got = torch.cat(got).cpu()
-    assert got.shape == want.shape
-    assert _rel(got, want) < 2e-5
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_wide_model_against_plain(folder, wide_plain, dtype, tol):
+    """Sums over 4,096 and 14,336 terms, a vocabulary of 128,256, 32 heads on 8."""
+    _batches_against_plain(folder, "wide", wide_plain, dtype, tol)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_wider_model_against_plain(wider_folder, wider_plain, dtype, tol):
+    """The widths of the 70B shape: sums over 8,192 and 28,672 terms, 64 heads on 8, the llama3
+    rule with its original length of 8,192."""
+    _batches_against_plain(wider_folder, "wider", wider_plain, dtype, tol)
 
 
 def test_wide_model_bfloat16_against_float32(folder):
+    """A drift report rather than a proof: twenty requests, alone and together, against the
+    engine's own float32 path (which the tests above compare with the plain implementation)."""
     import rbitnet_amd
     rng = np.random.default_rng(3)
     lengths = [700, 130, 65, 300, 1, 31, 64, 200, 90, 17, 450, 33, 257, 129, 5, 512, 77, 256, 40, 100]

@@ -104,10 +104,11 @@ def test_groups_by_need_and_readers():
             CacheRequest("state", state_shape=(3, 2), state_init=1.5)]
     c = Cache(reqs, 2, 64 * 8, torch.float32, "cpu", readers={2: 1})
     assert len(c.kv_groups) == 3 and len(c.state_groups) == 1
-    full = c.layer_kv[0][0]
-    assert full.layers == [0, 3] and c.layer_kv[3] == (full, 1)
-    assert c.layer_kv[2] == c.layer_kv[1]          # layer 2 reads layer 1's keys and values
-    assert c.layer_kv[4][0].k.shape == (1, 8, 1, PAGE_SIZE, 16)
+    kv = lambda l: next((g, i) for g, i in c.layer_groups[l] if g.kind == "kv")
+    full = kv(0)[0]
+    assert full.layers == [0, 3] and kv(3) == (full, 1)
+    assert kv(2) == kv(1)                            # layer 2 reads layer 1's keys and values
+    assert kv(4)[0].k.shape == (1, 8, 1, PAGE_SIZE, 16)
     with pytest.raises(CacheError, match="keeps none"):
         Cache([None, CacheRequest("kv", heads=1, head_dim=8)], 1, 64, torch.float32, "cpu", readers={1: 0})
 
@@ -125,7 +126,7 @@ def test_window_gives_pages_back_early():
         c.commit([s], [1])
         c.check()
     assert c.length(s) == 400 and g.table.pool.n_held <= 3     # a full group would hold 7
-    assert c.block_table(g, [s])[0][0] == 0                   # dead entries read as a valid page id
+    assert c.block_tables([s])[id(g)][0][0] == 0                   # dead entries read as a valid page id
     c.free_slot(s)
     assert g.table.pool.n_free == 6
 

@@ -17,7 +17,19 @@ def test_defaults_follow_the_reference():
                                  "intermediate_size": 100, "vocab_size": 50})
     assert cfg.num_key_value_heads == 4 and cfg.head_dim == 16
     assert cfg.rope_theta == 10000.0 and cfg.rms_norm_eps == 1e-5 and cfg.max_position_embeddings == 2048
-    assert cfg.rope_scaling is None and cfg.rope_style == "interleaved" and not cfg.tie_word_embeddings
+    assert cfg.rope_scaling is None and not cfg.tie_word_embeddings
+    # the pairing of the rotation: not said -> "half", the layout of weights stored under a
+    # config.json's own names; GGUF spellings in the weight file -> the reference's adjacent pairs
+    assert cfg.rope_style is None and cfg.effective_rope_style == "half"
+    assert cfg.to_spec().layers[0].mixer["position"]["style"] == "half"
+    hf = cfg.with_tensor_names(["model.layers.0.self_attn.q_proj.weight", "model.embed_tokens.weight"])
+    assert hf.effective_rope_style == "half"
+    gguf = cfg.with_tensor_names(["blk.0.attn_q.weight", "token_embd.weight"])
+    assert gguf.effective_rope_style == "interleaved" and "rope_style" in gguf.to_dict()
+    said = LlamaConfig.from_dict({"hidden_size": 64, "num_hidden_layers": 1, "num_attention_heads": 4,
+                                  "intermediate_size": 100, "vocab_size": 50, "rope_style": "half"})
+    assert said.with_tensor_names(["blk.0.attn_q.weight"]).effective_rope_style == "half"      # the key wins
+    assert "rope_style" not in cfg.to_dict()
 
 
 @pytest.mark.parametrize("key", ["hidden_size", "num_hidden_layers", "num_attention_heads", "intermediate_size",

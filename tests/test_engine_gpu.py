@@ -3,7 +3,8 @@ the last 32 tokens one by one, and batches of unequal lengths with slot reuse.""
 import pytest
 import torch
 
-from helpers import TOL, max_err, model_folder, plain_logits, tokens_for
+from helpers import (BF16_MAX_RATIO, BF16_RMS_RATIO, BF16_RMS_RATIO_FEW, CONFIGS, TOL, max_err, model_folder,
+                     plain_logits, plain_logits_rounded, rms_err, tokens_for)
 
 pytestmark = pytest.mark.gpu
 
@@ -124,3 +125,94 @@ def test_batch_that_shrinks_from_20_sequences_to_8(name, dtype):
         want = plain_logits(name, tuple(r))[prompt_len[i] - 1:]
         err = max_err(torch.cat(got[i]), want)
         assert err < TOL[dtype], f"{name} {dtype} request {i}: {err}"
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+def test_bfloat16_error_is_the_cost_of_rounding_and_no_more(name):
+    """The bound of 3e-2 on the bfloat16 engine is loose enough to let a systematic error of a
+    per cent pass.  What rounding to bfloat16 must cost is measured here by the plain
+    implementation rounding at the places where the engine stores bfloat16; the engine's error
+    against the exact logits may be that large and little more, as a root mean square over each
+    request's logits and at its worst logit.  Steps of at most 16 tokens fold the norms into the
+    products around them and round bf16(x * gain) instead of bf16(x * gain / rms): the same cost."""
+    cap = CONFIGS[name][0]["max_position_embeddings"]
+    eng = _engine(name, "bfloat16", max_tokens=1152)
+    for i, n in enumerate([40, 77, 150, 700]):
+        if n > cap:
+            continue
+        toks = tokens_for(name, n, 20 + i)
+        exact = plain_logits(name, tuple(toks))
+        rounded = plain_logits_rounded(name, tuple(toks))
+        slot = eng.alloc_slot()
+        got = eng.step([(slot, toks[:n - 8])], "all")
+        tail = torch.cat([eng.step([(slot, [t])], "last") for t in toks[n - 8:]])
+        eng.free_slot(slot)
+        head, last = slice(0, n - 8), slice(n - 8, n)
+        cost = rms_err(rounded[head], exact[head])
+        assert 1e-4 < cost < 1e-2                               # the plain implementation does round
+        assert rms_err(got, exact[head]) < BF16_RMS_RATIO * cost, f"{name} length {n}"
+        assert max_err(got, exact[head]) < BF16_MAX_RATIO * max_err(rounded[head], exact[head]), f"{name} length {n}"
+        assert rms_err(tail, exact[last]) < BF16_RMS_RATIO_FEW * rms_err(rounded[last], exact[last]), f"{name} length {n}"
+
+
+def test_folder_with_adjacent_pairs_and_permuted_rows_gives_the_same_logits(tmp_path):
+    """A weight file whose q and k rows were permuted for the reference's pairing of the rotation
+    (model.rs:122-136), read with "interleaved", against the same model un-permuted, read with
+    "half": the engine's two pairings are the same function."""
+    import json
+    import rbitnet_amd
+    from safetensors.torch import load_file, save_file
+    cfg = dict(CONFIGS["B"][0])
+    assert "rope_style" not in cfg
+    src = model_folder("B")
+    d = cfg["hidden_size"] // cfg["num_attention_heads"]
+    perm = torch.stack([torch.arange(d // 2), torch.arange(d // 2) + d // 2], dim=1).reshape(-1)
+    tensors = load_file(f"{src}/model.safetensors")
+    for key in list(tensors):
+        if key.endswith("q_proj.weight") or key.endswith("k_proj.weight"):
+            w = tensors[key]
+            tensors[key] = w.view(-1, d, w.shape[1])[:, perm, :].reshape(w.shape).contiguous()
+    dst = tmp_path / "permuted"
+    dst.mkdir()
+    save_file(tensors, str(dst / "model.safetensors"))
+    with open(dst / "config.json", "w") as f:
+        json.dump(dict(cfg, rope_style="interleaved"), f)
+    toks = tokens_for("B", 50, 3)
+    want = plain_logits("B", tuple(toks))
+    for folder in (src, str(dst)):
+        eng = rbitnet_amd.Engine.load_path(folder, dtype="float32", max_tokens=128)
+        slot = eng.alloc_slot()
+        assert max_err(eng.step([(slot, toks)], "all"), want) < TOL["float32"]
+        eng.free_slot(slot)
+
+
+def test_cache_for_a_configuration_with_a_very_long_context(tmp_path, monkeypatch, capfd):
+    """config.json files of real checkpoints allow 131,072 positions.  Without sizes from the caller
+    the cache is made for 8 such sequences if that fits the free memory, and for what fits
+    otherwise (with a message); a request beyond what fits ends with "context"; a size asked for
+    that does not fit is an error that says what would."""
+    import rbitnet_amd
+    from rbitnet_amd.errors import CacheError
+    cfg = dict(CONFIGS["A"][0], max_position_embeddings=131072)
+    folder = rbitnet_amd.write_random_model(str(tmp_path / "m"), cfg, seed=0, std=0.1)
+    per_token = 2 * cfg["num_hidden_layers"] * cfg["num_key_value_heads"] * 16 * 2        # k and v, bfloat16
+    eng = rbitnet_amd.Engine.load_path(folder)
+    assert eng.max_seq_len == 131072 and eng.cache.bytes() == 8 * 131072 * per_token
+    del eng
+    real = torch.cuda.mem_get_info
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda *a: (1 << 20, real(*a)[1]))    # 1 MiB is free
+    eng = rbitnet_amd.Engine.load_path(folder)
+    fits = int((1 << 20) * 0.9) // per_token // 64 * 64
+    assert eng.cache.bytes() == fits * per_token and eng.cache.token_capacity() == fits
+    assert "sized to the" in capfd.readouterr().err
+    (r,) = eng.generate([tokens_for("A", fits - 10, 1)], max_tokens=100, temperature=0.0, stop_token_ids=[])
+    assert r.finish_reason == "context" and len(r.tokens) == 11       # ten run, the last is only emitted
+    eng.cache.check()
+    with pytest.raises(CacheError, match="does not fit"):
+        rbitnet_amd.Engine.load_path(folder, max_tokens=1 << 20)
+    # the position limit of the reference (model.rs:221-223) still holds
+    small = rbitnet_amd.Engine.load_path(folder, max_seq_len=100, max_tokens=256)
+    slot = small.alloc_slot()
+    from rbitnet_amd.errors import InferenceError
+    with pytest.raises(InferenceError, match="max_seq"):
+        small.step([(slot, tokens_for("A", 101, 2))], "last")

@@ -114,8 +114,44 @@ def test_pages_running_out_end_with_context():
 
 def test_plan_batches():
     assert plan_batches([5, 5, 5], 10, 2, 100, 1000) == [[0, 1], [2]]
-    assert plan_batches([60, 60, 60], 10, 8, 1000, 4) == [[0, 1], [2]]       # 2 pages each, 4 pages
+    pages = lambda n: (n + 63) // 64 * 64
+    assert plan_batches([60, 60, 60], 10, 8, 1000, 256, pages) == [[0, 1], [2]]     # 128 tokens each of 256
+    assert plan_batches([60, 60, 60], 10, 8, 1000, 256) == [[0, 1, 2]]              # counted as they are: 70 each
     assert plan_batches([], 10, 2, 100, 10) == []
+
+
+def test_the_loop_asks_the_cache_in_tokens_only():
+    """The loop works with any cache that answers token_capacity / tokens_needed / can_grow:
+    here one without pages, which counts tokens as they are."""
+    class TokenCache:
+        def __init__(self, capacity):
+            self.capacity, self.lens, self.free = capacity, {}, [1, 0]
+
+        def token_capacity(self):
+            return self.capacity
+
+        def tokens_needed(self, n):
+            return n
+
+        def can_grow(self, slot, by=1):
+            return sum(self.lens.values()) + by <= self.capacity
+
+    eng = ScriptedEngine(max_batch=2, max_seq_len=1000)
+    eng.spec = type("S", (), {"stop_token_ids": [], "bos_token_id": None, "vocab_size": 16})()
+    cache = TokenCache(50)
+    eng.cache = cache
+    eng.alloc_slot = lambda: (cache.lens.__setitem__(cache.free[-1], 0), cache.free.pop())[1]
+    eng.free_slot = lambda s: (cache.lens.pop(s), cache.free.append(s))
+    def step(entries, want):
+        for s, t in entries:
+            cache.lens[s] += len(t)
+        return [(t[-1] + 1) % 16 for _, t in entries]
+    eng.step = step
+    rs = generate(eng, [[1] * 20, [2] * 20], max_tokens=100, temperature=0.0)
+    # each may come to 120 tokens and is planned with all 50: one after the other, each until 50 are held
+    assert [r.finish_reason for r in rs] == ["context", "context"]
+    assert [len(r.tokens) for r in rs] == [31, 31]
+    assert not cache.lens
 
 
 def test_uniform_is_keyed_by_seed_sequence_and_count():
@@ -129,9 +165,9 @@ def test_uniform_is_keyed_by_seed_sequence_and_count():
 def test_decode_attention_split_rule(monkeypatch):
     """How many workgroups share the pages of one (sequence, kv head) in decode attention:
     none up to 15 pages, two from 16 pages, four from 32 and so on to at most 16, and never more than gives
-    every compute unit about one workgroup; an environment variable overrides the rule."""
+    every compute unit about one workgroup; a module attribute overrides the rule for tests."""
+    from rbitnet_amd.engine import context
     from rbitnet_amd.engine.context import decode_splits, split_bucket
-    monkeypatch.delenv("RBITNET_DECODE_SPLITS", raising=False)
     assert [split_bucket(n) for n in (1, 64, 960, 961, 1024, 2047, 2049, 4096, 8192, 10 ** 6)] == \
         [1, 1, 1, 2, 2, 4, 4, 8, 16, 16]
     assert split_bucket(0) == 1
@@ -140,5 +176,6 @@ def test_decode_attention_split_rule(monkeypatch):
     assert decode_splits(1, 8, split_bucket(4096)) == 8
     assert decode_splits(64, 8, split_bucket(65536)) == 1
     assert decode_splits(1, 1, 16) == 16
-    monkeypatch.setenv("RBITNET_DECODE_SPLITS", "3")
+    assert decode_splits(8, 8, 16, n_compute_units=128) == 2     # a smaller GPU
+    monkeypatch.setattr(context, "FORCED_DECODE_SPLITS", 3)
     assert decode_splits(64, 8, 1) == 3

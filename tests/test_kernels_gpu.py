@@ -74,14 +74,14 @@ def test_gemm_bf16(lib, m, n, k):
 @pytest.mark.parametrize("m", [1, 8, 20, 64, 100, 260])
 @pytest.mark.parametrize("ff,k", [(16, 64), (336, 192), (8208, 136), (17000 // 16 * 16, 72)])
 def test_gemm_bf16_gated(lib, m, ff, k):
-    from rbitnet_amd.parts.linear import pack_gate_up
+    from helpers import interleave_gate_up
     g = torch.Generator().manual_seed(m + ff)
     x = torch.randn(m, k, generator=g).bfloat16()
     wg = (torch.randn(ff, k, generator=g) * 0.3).bfloat16()
     wu = (torch.randn(ff, k, generator=g) * 0.3).bfloat16()
     gate = x.double() @ wg.double().T
     want = gate / (1 + torch.exp(-gate)) * (x.double() @ wu.double().T)
-    packed = pack_gate_up(wg, wu, True).to(DEV)
+    packed = interleave_gate_up(wg, wu).to(DEV)
     out = torch.full((m, ff), float("nan"), device=DEV, dtype=torch.bfloat16)
     lib.gemm_bf16(x.to(DEV), packed, out, 1)
     assert _rel(out, want) < 1e-2
@@ -109,7 +109,7 @@ def test_gemm_bf16_tiles_loaded_straight_into_lds(lib, m, n, k, gated):
     tiles than of 256-row ones (5 x 45 = 225 against 5 x 56 = 280, and 4 x 180 against 4 x 224).
     The last five are tiles too few for a round whose K is cut: 48 tiles of 256 x 128 in 4 slices,
     85 in 2, 105 tiles of 192 x 256 in 2, 96 of 256 x 256 in 2, and 192 tiles of 192 x 256 uncut."""
-    from rbitnet_amd.parts.linear import pack_gate_up
+    from helpers import interleave_gate_up
     g = torch.Generator().manual_seed(m + n + k)
     x = torch.randn(m, k, generator=g).bfloat16()
     if gated:
@@ -119,7 +119,7 @@ def test_gemm_bf16_tiles_loaded_straight_into_lds(lib, m, n, k, gated):
         gate = x.double() @ wg.double().T
         want = gate / (1 + torch.exp(-gate)) * (x.double() @ wu.double().T)
         out = torch.full((m, ff), float("nan"), device=DEV, dtype=torch.bfloat16)
-        lib.gemm_bf16(x.to(DEV), pack_gate_up(wg, wu, True).to(DEV), out, 1)
+        lib.gemm_bf16(x.to(DEV), interleave_gate_up(wg, wu).to(DEV), out, 1)
         assert _rel(out, want) < 1e-2
     else:
         w = torch.randn(n, k, generator=g).bfloat16()
@@ -542,13 +542,13 @@ def test_gemm_bf16_17_to_64_tokens(lib, m, n, k, epi):
     g = torch.Generator().manual_seed(m * 3 + n)
     a = torch.randn(m, k, generator=g).bfloat16()
     if epi:
-        from rbitnet_amd.parts.linear import pack_gate_up
+        from helpers import interleave_gate_up
         ff = n // 2
         wg = (torch.randn(ff, k, generator=g) * 0.3).bfloat16()
         wu = (torch.randn(ff, k, generator=g) * 0.3).bfloat16()
         gate = a.double() @ wg.double().T
         want = gate / (1 + torch.exp(-gate)) * (a.double() @ wu.double().T)
-        w = pack_gate_up(wg, wu, True)
+        w = interleave_gate_up(wg, wu)
         out = torch.full((m, ff), float("nan"), device=DEV, dtype=torch.bfloat16)
         tol = 1e-2
     else:
@@ -587,7 +587,7 @@ def test_gemm_bf16_few_tokens_folds_sum_and_norm(lib, m, n, k):
     keeps the tokens in registers (more than 8192 rows of W, K a multiple of 512 up to 4096).
     The matrix cores see bf16(x * gain), which the first reference repeats; the second is the
     norm as its own kernel computes it, rounded after the root."""
-    from rbitnet_amd.parts.linear import pack_gate_up
+    from helpers import interleave_gate_up
     assert lib.gemm_bf16_few_ok(m, n, k)
     g = torch.Generator().manual_seed(m * 11 + n + k)
     eps = 1e-3
@@ -637,7 +637,7 @@ def test_gemm_bf16_few_tokens_folds_sum_and_norm(lib, m, n, k):
         gate = (gained[:m].double() @ wg.double().T) * scale
         want = gate / (1 + torch.exp(-gate)) * ((gained[:m].double() @ wu.double().T) * scale)
         out = torch.full((m, ff), float("nan"), device=DEV, dtype=torch.bfloat16)
-        lib.gemm_bf16_few(gained[:m].contiguous().to(DEV), pack_gate_up(wg, wu, True).to(DEV), out, 1,
+        lib.gemm_bf16_few(gained[:m].contiguous().to(DEV), interleave_gate_up(wg, wu).to(DEV), out, 1,
                           squares=squares[:m].contiguous().to(DEV), eps=eps)
         assert _rel(out, want) < 1e-2
 

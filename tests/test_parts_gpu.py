@@ -10,7 +10,7 @@ import torch
 import plain_llama as P
 from rbitnet_amd.cache import Cache
 from rbitnet_amd.config.spec import LayerSpec, ModelSpec, PartSpec
-from rbitnet_amd.engine.context import StepContext
+from rbitnet_amd.engine.context import StepBatch, StepContext
 from rbitnet_amd.parts import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register_mixer
 
 pytestmark = pytest.mark.gpu
@@ -44,9 +44,7 @@ def _ctx_and_cache(part, past, tokens_per_seq, dtype):
 def _step(cache, slots, q_lens):
     past = [cache.length(s) for s in slots]
     cache.reserve(slots, q_lens)
-    tables = {id(g): cache.block_table(g, slots) for g in cache.kv_groups}
-    ctx = StepContext(DEV, slots, past, [[0] * q for q in q_lens], [], tables)
-    return ctx
+    return StepContext.for_batch(DEV, StepBatch(slots, past, [[0] * q for q in q_lens], [], cache.block_tables(slots)))
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-6), (torch.bfloat16, 8e-3)])
@@ -260,6 +258,115 @@ def test_toy_mixer_and_mixed_layers(dtype, tol):
     eng.cache.check()
     # the windowed group gave pages back while the long sequence ran
     assert eng.cache.kv_groups[0].table.pool.n_free == eng.cache.n_pages
+
+
+class ScaledDecayMixer(Part):
+    """The state mixer again, with two things more: its input is weighted per token by an array
+    that the step layout carries for it (declared below with `declare_step_array`, computed on the
+    host from the batch for every step), and with one token per sequence its forward only launches
+    device work, so that the decode step it is part of can be captured:
+        s_t = a * s_{t-1} + h_t / (1 + pos_t / 8),  out_t = W s_t."""
+    graph_safe = True
+
+    def __init__(self, params, env):
+        self.env, self.a, self.hidden = env, float(params["decay"]), env.hidden_size
+
+    def tensor_specs(self):
+        return {"mix.weight": TensorSpec((self.hidden, self.hidden))}
+
+    def load(self, tensors):
+        self.w = tensors["mix.weight"]
+
+    def cache_request(self):
+        return CacheRequest("state", state_shape=(self.hidden,), state_init=0.0)
+
+    def forward(self, h, ctx, view):
+        hf = h.float() * ctx.extra["toy_token_weight"][:, None]
+        if ctx.max_q_len == 1:                               # one token each: device work only
+            idx = ctx.slots.long()
+            s = self.a * view.state.index_select(0, idx) + hf
+            view.state.index_copy_(0, idx, s)
+            return s @ self.w.float().T
+        out = torch.empty_like(hf)
+        at = 0
+        for slot, n in zip(ctx.host_slots, ctx.q_lens):      # the host knows the layout: nothing is read back
+            s = view.state[slot]
+            for t in range(at, at + n):
+                s = self.a * s + hf[t]
+                out[t] = s
+            view.state[slot] = s
+            at += n
+        return out @ self.w.float().T
+
+
+def _toy_token_weight(batch):
+    import numpy as np
+    pos = np.concatenate([p + np.arange(len(t)) for p, t in zip(batch.past_lens, batch.tokens)])
+    return (1.0 / (1.0 + pos / 8.0)).astype(np.float32)
+
+
+def test_toy_mixer_with_a_step_array_of_its_own_runs_captured():
+    """One declaration gives a part a per-step array, in steps launched kernel by kernel and in the
+    captured decode step alike; the state is updated once per step there too (the step that runs
+    before the capture counts, the capture itself executes nothing)."""
+    import rbitnet_amd
+    from rbitnet_amd.engine.context import declare_step_array, forget_step_array
+    declare_step_array("toy_token_weight", "float32", lambda n_seqs, n_tokens: n_tokens, _toy_token_weight)
+    try:
+        _run_scaled_decay_model()
+    finally:
+        forget_step_array("toy_token_weight")
+
+
+def _run_scaled_decay_model():
+    import rbitnet_amd
+    from rbitnet_amd.engine.model import expected_tensors
+    from rbitnet_amd.weights import random_tensors
+    register_mixer("toy_scaled_decay", ScaledDecayMixer)
+    hidden, vocab = 64, 80
+    norm = PartSpec("rmsnorm", {"size": hidden, "eps": 1e-5})
+    layers = [LayerSpec(f"blocks.{i}", "prenorm", PartSpec("toy_scaled_decay", {"decay": 0.6 + 0.1 * i}),
+                        PartSpec("swiglu", {"intermediate_size": 96}), norm, norm) for i in range(2)]
+    spec = ModelSpec(architecture="ToyForTests", hidden_size=hidden, vocab_size=vocab, max_positions=256,
+                     embedding_name="embed.weight", layers=layers, final_norm=norm,
+                     final_norm_name="final_norm.weight", head_name="head.weight")
+    tensors = dict(random_tensors(expected_tensors(spec), seed=9, std=0.2, norm_std=0.05, dtype=torch.bfloat16))
+
+    def plain(tokens):
+        w = {k: v.double() for k, v in tensors.items()}
+        x = P.embedding(w["embed.weight"], tokens)
+        for i, layer in enumerate(spec.layers):
+            pre = layer.prefix
+            h = P.rmsnorm(x, w[f"{pre}.input_layernorm.weight"], 1e-5)
+            s, rows = torch.zeros(hidden, dtype=D64), []
+            for t in range(h.shape[0]):
+                s = layer.mixer["decay"] * s + h[t] / (1.0 + t / 8.0)
+                rows.append(s)
+            x = x + P.linear(torch.stack(rows), w[f"{pre}.self_attn.mix.weight"])
+            h2 = P.rmsnorm(x, w[f"{pre}.post_attention_layernorm.weight"], 1e-5)
+            x = x + P.swiglu(h2, w[f"{pre}.mlp.gate_proj.weight"], w[f"{pre}.mlp.up_proj.weight"],
+                             w[f"{pre}.mlp.down_proj.weight"])
+        return P.linear(P.rmsnorm(x, w["final_norm.weight"], 1e-5), w["head.weight"])
+
+    eng = rbitnet_amd.Engine.from_spec(spec, tensors, dtype="float32", max_tokens=64 * 4, max_batch=2)
+    assert eng.use_graphs and not eng.cache.kv_groups
+    g = torch.Generator().manual_seed(3)
+    seqs = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in (30, 12)]
+    want = [plain(s) for s in seqs]
+    for graphs in (True, False):
+        eng.use_graphs = graphs
+        slots = [eng.alloc_slot() for _ in seqs]
+        cut = [len(s) - 6 for s in seqs]
+        logits = eng.step([(sl, s[:c]) for sl, s, c in zip(slots, seqs, cut)], "last")
+        for i, (c, w) in enumerate(zip(cut, want)):
+            assert _rel(logits[i:i + 1], w[c - 1:c]) < 2e-5
+        for j in range(6):                                   # decode steps: the first runs before the capture
+            eng.decode_step(slots, [s[c + j] for s, c in zip(seqs, cut)])
+            for i, (c, w) in enumerate(zip(cut, want)):
+                assert _rel(eng.last_decode_logits[i:i + 1], w[c + j:c + j + 1]) < 2e-5, (graphs, j, i)
+        for sl in slots:
+            eng.free_slot(sl)
+    assert len(eng._graphs) == 1
 
 
 # ---------------------------------------------------------------------------- other toy parts

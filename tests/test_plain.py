@@ -104,15 +104,82 @@ def test_llama3_scaling_branches():
     assert torch.all(got[1:] < got[:-1])                                        # still monotone
     one = dict(sc, factor=1.0)
     assert torch.allclose(P.rope_inv_freq(d, theta, one), plain)
-    # continuous at both boundaries: a wavelength just inside the middle range gives nearly
-    # the value of the branch next to it
-    for boundary, neighbour in ((32 / 4.0, 1.0), (32 / 1.0, 1 / 8.0)):
-        inv_b = 2 * math.pi / boundary
-        s = (32 / boundary - 1.0) / (4.0 - 1.0)
-        assert abs(((1 - s) / 8.0 + s) - neighbour) < 1e-12
     # the engine's table builder is a different piece of code and must agree
     from rbitnet_amd.parts.position import rope_inverse_frequencies
     assert torch.allclose(rope_inverse_frequencies(d, theta, sc), got, rtol=1e-14)
+
+
+def test_llama3_middle_range_is_the_one_affine_blend():
+    """Between the two boundaries the scaled frequency divided by the unscaled one is an affine
+    function of the frequency (the blend is linear in original / wavelength) that meets the
+    branch on either side without a jump.  An affine function with both ends fixed is unique,
+    so these three properties are the rule; a blend with its two weights swapped, or one linear
+    in the wavelength, fails.  The frequencies lie 0.45 % apart here (head size 4096), so that
+    some fall just inside either boundary."""
+    d, theta = 4096, 10000.0
+    orig, low, high, factor = 32, 1.0, 4.0, 8.0
+    sc = {"rope_type": "llama3", "factor": factor, "low_freq_factor": low, "high_freq_factor": high,
+          "original_max_position_embeddings": orig}
+    plain = P.rope_inv_freq(d, theta, None)
+    got = P.rope_inv_freq(d, theta, sc)
+    ratio = got / plain
+    lam = 2 * math.pi / plain
+    step = theta ** (2.0 / d) - 1.0                                    # neighbouring wavelengths differ by this
+    assert step < 0.005
+    short, long_ = lam < orig / high, lam > orig / low
+    mid = ~short & ~long_
+    assert int(mid.sum()) > 250 and short.any() and long_.any()
+    assert torch.all(ratio[short] == 1.0) and torch.allclose(ratio[long_], torch.full_like(ratio[long_], 1 / factor))
+    idx = torch.nonzero(mid).flatten()
+    first, last = int(idx[0]), int(idx[-1])
+    # no jump at the short-wave boundary: the first middle frequency is nearly unscaled ...
+    assert abs(float(ratio[first]) - 1.0) < 7.0 / 6.0 * step + 1e-12
+    # ... nor at the long-wave boundary: the last one is nearly divided by the factor
+    assert abs(float(ratio[last]) - 1.0 / factor) < (1 - 1 / factor) / (high - low) * step + 1e-12
+    # strictly between, falling as the waves get longer
+    assert torch.all(ratio[idx][1:] < ratio[idx][:-1]) and ratio[last] > 1 / factor and ratio[first] < 1.0
+    # affine in the frequency: equal slopes between any neighbours
+    f, r = plain[idx], ratio[idx]
+    slopes = (r[1:] - r[:-1]) / (f[1:] - f[:-1])
+    assert float((slopes.max() - slopes.min()) / slopes.mean().abs()) < 1e-9
+    # the slope itself, from the two fixed ends: (1 - 1/factor) / (f(orig/high) - f(orig/low))
+    want_slope = (1 - 1 / factor) / (2 * math.pi * high / orig - 2 * math.pi * low / orig)
+    assert abs(float(slopes.mean()) / want_slope - 1.0) < 1e-9
+    # the shape the large models use (head size 128, theta 5e5, original length 8192): the same
+    # affine map, and the engine's table builder agrees on every frequency
+    sc2 = dict(sc, original_max_position_embeddings=8192)
+    p2, g2 = P.rope_inv_freq(128, 500000.0, None), P.rope_inv_freq(128, 500000.0, sc2)
+    lam2 = 2 * math.pi / p2
+    m2 = (lam2 >= 8192 / high) & (lam2 <= 8192 / low)
+    assert int(m2.sum()) >= 6
+    affine = 1 / factor + (1 - 1 / factor) * (8192 * p2[m2] / (2 * math.pi) - low) / (high - low)
+    assert torch.allclose(g2[m2] / p2[m2], affine, rtol=1e-12)
+    from rbitnet_amd.parts.position import rope_inverse_frequencies
+    assert torch.allclose(rope_inverse_frequencies(128, 500000.0, sc2), g2, rtol=1e-14)
+    assert torch.allclose(rope_inverse_frequencies(d, theta, sc), got, rtol=1e-14)
+
+
+def test_half_pairing_of_a_whole_model_equals_adjacent_pairs_on_permuted_rows():
+    """The two pairings of the rotation differ by a permutation of the rows of Wq and Wk inside
+    every head (scores are dot products, which no common permutation changes): a model read with
+    "half" and the same model with these rows permuted and read with adjacent pairs, as the
+    reference rotates (model.rs:122-136), give the same logits."""
+    m = P.PlainLlama.from_folder(model_folder("B"))
+    assert m.style == "half"                                             # no key in config.json: names decide
+    toks = [5, 6, 7, 300, 2, 9]
+    d = m.head_dim
+    perm = torch.stack([torch.arange(d // 2), torch.arange(d // 2) + d // 2], dim=1).reshape(-1)   # new[2i] = old[i]
+    z = copy.copy(m)
+    z.w = dict(m.w)
+    z.style = "interleaved"
+    for il in range(m.n_layer):
+        for name, heads in (("q_proj", m.n_head), ("k_proj", m.n_kv)):
+            key = f"model.layers.{il}.self_attn.{name}.weight"
+            w = m.w[key].view(heads, d, -1)
+            z.w[key] = w[:, perm, :].reshape(heads * d, -1)
+    assert torch.allclose(z.logits(toks), m.logits(toks), atol=1e-12)
+    z.style = "half"
+    assert not torch.allclose(z.logits(toks), m.logits(toks), atol=1e-6)         # the pairing matters
 
 
 def test_attention_reduces_to_library_attention():
