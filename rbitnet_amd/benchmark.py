@@ -143,8 +143,11 @@ def main(argv=None) -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    ap.add_argument("--points", default="1,64", help="batch sizes of the extra decode points")
     ap.add_argument("--model", default="llama3_8b", choices=sorted(MODELS),
                     help="shape to measure (default: the baseline's configs[2])")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                    help="length of the one prompt whose prefill is timed")
     ap.add_argument("--prompt-len", default=str(PROMPT_LEN),
                     help="context at which decoding starts; LO,HI draws unequal lengths uniformly")
     args = ap.parse_args(argv)
@@ -167,11 +170,15 @@ def main(argv=None) -> int:
         cfg["num_hidden_layers"] = args.layers
     layers = cfg["num_hidden_layers"]
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
-    max_batch = max(args.batch, 1 if args.no_points else 64)
+    max_batch = max([args.batch] + ([] if args.no_points else [int(v) for v in args.points.split(",") if v]))
     ctx_cap = longest + max(NEW_TOKENS, args.steps + args.warmup) + 64
-    max_tokens = max(max_batch * ctx_cap, PREFILL_TOKENS + 64)
+    prefill_tokens = args.prefill_tokens
+    max_tokens = max(max_batch * ctx_cap, prefill_tokens + 64)
+    max_seq_len = max(ctx_cap, prefill_tokens + 64)
+    # contexts beyond what the named configuration allows are measured with its limit raised
+    cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], max_seq_len)
     engine = Engine.random(cfg, seed=0, dtype=dtype, std=0.02, norm_std=0.0, max_batch=max_batch,
-                                       max_tokens=max_tokens, max_seq_len=max(ctx_cap, PREFILL_TOKENS + 64))
+                           max_tokens=max_tokens, max_seq_len=max_seq_len)
     _sync()
 
     dt, ctx_mean = decode_run(engine, args.batch, args.steps, args.warmup, prompt_len=prompt_len)
@@ -206,7 +213,7 @@ def main(argv=None) -> int:
         # ---- prefill of one prompt of 2,048 tokens
         import numpy as np
         rng = np.random.default_rng(1)
-        prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=PREFILL_TOKENS)]
+        prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=prefill_tokens)]
         times = []
         for i in range(PREFILL_RUNS + 1):
             slot = engine.alloc_slot()
@@ -218,16 +225,19 @@ def main(argv=None) -> int:
             engine.free_slot(slot)
         pt = sorted(times[1:])[len(times[1:]) // 2]           # the median; the first run warms up
         layer_flops, head_flops = matmul_flops_per_token(cfg)
-        attn_flops = 4.0 * cfg["num_attention_heads"] * d * layers * (PREFILL_TOKENS * (PREFILL_TOKENS + 1) / 2.0)
-        flops = layer_flops * PREFILL_TOKENS + head_flops * 1 + attn_flops
-        out["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
+        attn_flops = 4.0 * cfg["num_attention_heads"] * d * layers * (prefill_tokens * (prefill_tokens + 1) / 2.0)
+        flops = layer_flops * prefill_tokens + head_flops * 1 + attn_flops
+        out["prefill"] = {"value": round(prefill_tokens / pt, 1), "tokens": prefill_tokens, "ms": round(pt * 1e3, 3),
                           "frac": round(flops / pt / PEAK_FLOPS[args.dtype], 4), "runs": PREFILL_RUNS,
                           "min_ms": round(min(times[1:]) * 1e3, 3)}
-        points = {}
-        for b in (1, 64):                 # the same prompts and number of steps as the headline batch
-            dtb, _ = decode_run(engine, b, args.steps, args.warmup, seed=b, prompt_len=prompt_len)
+        points, fracs = {}, {}
+        for b in [int(v) for v in args.points.split(",") if v]:      # the same prompts and number of steps as the headline batch
+            dtb, ctx_b = decode_run(engine, b, args.steps, args.warmup, seed=b, prompt_len=prompt_len)
             points[f"decode_b{b}"] = round(b * args.steps / dtb, 2)
+            fracs[f"decode_b{b}"] = round((engine.model.weight_bytes() + b * ctx_b * kv_bytes_per_token)
+                                          / (dtb / args.steps) / PEAK_HBM, 4)
         out["points"] = points
+        out["points_roofline_frac"] = fracs      # as `roofline.frac`, for each point
         # the practical ceilings of this GPU, for reading the fractions above
         out["probe"] = probe(engine.lib, engine.device)
 

@@ -554,6 +554,7 @@ static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, in
 //   cfg 6: 192 x 256 (8 waves)        ... when that fills the last round of workgroups better
 //   cfg 5: 128 x 128 (4 waves, 2 workgroups per compute unit)
 //   cfg 7: 128 rows of W x 64 tokens, 3 stages deep    up to 512 tokens, when cfg 5 has < 256 tiles
+//   cfg 10, 13: its variants for wide gated products of at most 64 tokens (see plan_tiles)
 //   cfg 1..3: tiles staged through registers, for K that is no multiple of 64 (more than 64 tokens)
 // Without K slices a product of 128 tokens by 4096 rows ran on 32 of the 256 compute units and
 // took as long as one of 768 tokens (K = 14336: 194 us; 41 us with 4 slices of 64-token tiles).
@@ -635,6 +636,14 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   }
   if (m > 64 && t192r >= 176 && t192r <= 256) return {6, 1};
   if (m > 64 && (t128 >= 256 || m > 512)) return {5, epilogue ? 1 : k_slices(t128, k, 512, k / (4 * m))};
+  // A gated product of at most 64 tokens cannot cut K and streams W from too few workgroups to
+  // hide anything (28,672 rows: 224 tiles of 128): tiles of 64 rows, four stages deep, two to a
+  // compute unit, up to 24 tokens (17 tokens: 45 us against 50), and K tiles of 128 (256 bytes a
+  // row and load) beyond (64 tokens: 49.2 against 50.8).
+  if (m <= 64 && epilogue == 1 && n >= 16384) {
+    if (m <= 24) return {10, 1};
+    if (k % 128 == 0) return {13, 1};
+  }
   return {7, epilogue ? 1 : k_slices(t64, k, 256, k / (8 * m))};
 }
 
@@ -650,6 +659,8 @@ static int launch_planned(const bf16_t* x, const bf16_t* w, void* c, float* work
     case 8: return launch_dma_cfg<256, 128, 64, 64, 64, 3, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
     case 9: return launch_dma_cfg<320, 256, 160, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
     case 7: return launch_dma_cfg<128, 64, 32, 64, 64, 3, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
+    case 10: return launch_dma_cfg<64, 64, 32, 32, 64, 4, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
+    case 13: return launch_dma_cfg<128, 64, 32, 64, 128, 3, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
     case 6: return launch_dma_cfg<192, 256, 96, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
     case 5: return launch_dma_cfg<128, 128, 64, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
     case 4: return launch_dma_cfg<256, 256, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);

@@ -64,18 +64,25 @@ class KernelTimes:
     launched kernel by kernel instead of replayed as a graph, so that every launch can be timed);
     the table goes to standard error when the process ends, or to whoever calls `report()`."""
 
-    def __init__(self) -> None:
+    def __init__(self, by_shape: bool = False) -> None:
+        """by_shape (RBITNET_KERNEL_TIMES=shapes): a row per wrapper and shapes of its first two
+        tensors, so that the products of a layer can be told apart."""
+        self.by_shape = by_shape
         self.events: Dict[str, List[Tuple[torch.cuda.Event, torch.cuda.Event]]] = {}
 
     def wrap(self, name: str, fn):
         def timed(*args, **kwargs):
+            key = name
+            if self.by_shape:
+                shapes = [tuple(a.shape) for a in args if hasattr(a, "shape")][:2]
+                key = f"{name} " + " x ".join("[" + ",".join(str(d) for d in sh) + "]" for sh in shapes)
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record()
             try:
                 return fn(*args, **kwargs)
             finally:
                 end.record()
-                self.events.setdefault(name, []).append((start, end))
+                self.events.setdefault(key, []).append((start, end))
         return timed
 
     def totals(self) -> Dict[str, Tuple[int, float]]:
@@ -89,9 +96,10 @@ class KernelTimes:
     def report(self) -> str:
         totals = self.totals()
         whole = sum(ms for _, ms in totals.values()) or 1.0
-        lines = [f"{'kernel':32} {'calls':>8} {'total ms':>10} {'mean us':>9} {'share':>6}"]
+        width = max([32] + [len(name) for name in totals])
+        lines = [f"{'kernel':{width}} {'calls':>8} {'total ms':>10} {'mean us':>9} {'share':>6}"]
         for name, (calls, ms) in sorted(totals.items(), key=lambda kv: -kv[1][1]):
-            lines.append(f"{name:32} {calls:8d} {ms:10.3f} {ms * 1e3 / max(1, calls):9.1f} {ms / whole:6.1%}")
+            lines.append(f"{name:{width}} {calls:8d} {ms:10.3f} {ms * 1e3 / max(1, calls):9.1f} {ms / whole:6.1%}")
         return "\n".join(lines)
 
 
@@ -147,8 +155,8 @@ class Kernels:
         L.rb_sample_workspace_bytes.restype = _I
         self.page_size = int(L.rb_page_size())
         self.times: Optional[KernelTimes] = None
-        if os.environ.get("RBITNET_KERNEL_TIMES", "") in ("1", "true", "yes"):
-            self.times = KernelTimes()
+        if os.environ.get("RBITNET_KERNEL_TIMES", "") in ("1", "true", "yes", "shapes"):
+            self.times = KernelTimes(by_shape=os.environ["RBITNET_KERNEL_TIMES"] == "shapes")
             for name in TIMED_OPS:
                 setattr(self, name, self.times.wrap(name, getattr(self, name)))
             atexit.register(lambda: print(self.times.report(), file=sys.stderr, flush=True))
