@@ -36,6 +36,11 @@ def split_bucket(max_kv_len: int) -> int:
     return bucket
 
 
+def bucket_max_pages(bucket: int) -> int:
+    """The most pages a sequence can hold while its batch is in this bucket (None: no bound)."""
+    return None if bucket >= 16 else 16 * bucket - 1
+
+
 def decode_splits(n_seqs: int, n_kv_heads: int, bucket: int = 16, n_compute_units: int = 256) -> int:
     """Into how many workgroups the pages of one (sequence, kv head) are dealt in decode
     attention: what the context length asks for (`split_bucket`), but no more than gives

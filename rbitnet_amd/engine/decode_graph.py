@@ -16,7 +16,7 @@ from typing import Optional
 
 import torch
 
-from .context import StepBatch, StepContext
+from .context import StepBatch, StepContext, bucket_max_pages
 
 
 class DecodeGraph:
@@ -28,7 +28,12 @@ class DecodeGraph:
     def __init__(self, engine, n_seqs: int, bucket: int = 16):
         self.engine = engine
         self.n_seqs = n_seqs
-        width = max(1, engine.cache.pages_per_sequence(engine.max_seq_len))
+        # page tables as wide as a sequence of this graph can need: no longer than the engine
+        # allows, than the cache has pages, or than the contexts of this split bucket reach
+        width = min(engine.cache.pages_per_sequence(engine.max_seq_len), engine.cache.n_pages)
+        if bucket_max_pages(bucket) is not None:
+            width = min(width, bucket_max_pages(bucket))
+        width = max(1, width)
         self.ctx = StepContext(engine.device, n_seqs, n_seqs, n_seqs,
                                {key: width for key in engine.cache.group_keys()}, bucket=bucket,
                                n_compute_units=engine.lib.n_compute_units)

@@ -86,6 +86,7 @@ class Engine:
         per_token = cache_bytes_per_token(model.cache_requests(), model.dtype)
         fits = 1 << 40
         if per_token > 0 and model.device.type == "cuda":
+            torch.cuda.empty_cache()          # what loading held for a moment counts as free
             free, _ = torch.cuda.mem_get_info(model.device)
             fits = int(free * CACHE_MEMORY_FRACTION) // per_token // PAGE_SIZE * PAGE_SIZE
         if max_tokens is not None:

@@ -171,6 +171,11 @@ def test_decode_attention_split_rule(monkeypatch):
     assert [split_bucket(n) for n in (1, 64, 960, 961, 1024, 2047, 2049, 4096, 8192, 10 ** 6)] == \
         [1, 1, 1, 2, 2, 4, 4, 8, 16, 16]
     assert split_bucket(0) == 1
+    # a bucket's contexts reach so many pages and no more (the captured step's page tables are that wide)
+    from rbitnet_amd.engine.context import bucket_max_pages
+    for b in (1, 2, 4, 8):
+        assert split_bucket(64 * bucket_max_pages(b)) == b and split_bucket(64 * bucket_max_pages(b) + 1) == 2 * b
+    assert bucket_max_pages(16) is None
     assert decode_splits(8, 8, split_bucket(600)) == 1
     assert decode_splits(8, 8, split_bucket(4096)) == 4          # 256 // (8 * 8)
     assert decode_splits(1, 8, split_bucket(4096)) == 8
