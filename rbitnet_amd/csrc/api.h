@@ -52,17 +52,22 @@ int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dty
 //               (16 gate rows, then the 16 up rows of the same columns); the result is
 //               silu(gate) * up, [M, N/2]
 // K must be a multiple of 8 (rows 16-byte aligned).
+// w_layout says how W is stored.  0: N rows of K values.  1: fragment-major (K % 64 == 0 and
+// N % 16 == 0 only): blocks of 16 rows x 32 depth values, 1 KB each, in the order [N / 16][K / 32];
+// inside a block, the value of row r and depth d lies at 8 * (16 * (d / 8) + r) + d % 8.  A wave
+// then reads 1 KB in a row per load, and a product of few tokens streams W with non-temporal
+// loads: 6.0-6.8 TB/s instead of 5.3-5.8.  rb_place_rows writes either layout.
 // workspace: rb_gemm_workspace_floats(m, n, k, epilogue) floats (0: none, null allowed); contents do
 // not matter before or after.
 long long rb_gemm_workspace_floats(int m, int n, int k, int epilogue);
-int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out, int epilogue, int m, int n, int k,
+int rb_gemm_bf16(const void* a, const void* w, int w_layout, void* c, int dtype_out, int epilogue, int m, int n, int k,
                  float* workspace, void* stream);
 
 // The plain product (float32, epilogue 0) as the terms that the K slices of its kernel computed:
 // terms [rb_gemm_bf16_terms_count(m, n, k), M, N], to be added up in their order.  One term is
 // the product itself.  For a caller that adds them to something else anyway.
 int rb_gemm_bf16_terms_count(int m, int n, int k);
-int rb_gemm_bf16_terms(const void* a, const void* w, float* terms, int m, int n, int k, void* stream);
+int rb_gemm_bf16_terms(const void* a, const void* w, int w_layout, float* terms, int m, int n, int k, void* stream);
 
 // The same product for 1..16 tokens with what stands before and after it in a decode step folded
 // in, so that no kernel runs between the products.  rb_gemm_bf16_few_ok: whether it takes these
@@ -74,9 +79,9 @@ int rb_gemm_bf16_terms(const void* a, const void* w, float* terms, int m, int n,
 //   epilogue 0, 1: as above.  2: C (float32) += product.  3: as 2, and for the norm that follows
 //     gained [M, N] = bf16(C * gain), squares_out [M, ceil(N / 16)] = sums of C^2 over 16 columns.
 int rb_gemm_bf16_few_ok(int m, int n, int k);
-int rb_gemm_bf16_few(const void* a, const float* squares_in, float eps, const int32_t* rows, const void* w, void* c,
-                     int dtype_out, int epilogue, const float* gain, void* gained, float* squares_out, int m, int n,
-                     int k, void* stream);
+int rb_gemm_bf16_few(const void* a, const float* squares_in, float eps, const int32_t* rows, const void* w,
+                     int w_layout, void* c, int dtype_out, int epilogue, const float* gain, void* gained,
+                     float* squares_out, int m, int n, int k, void* stream);
 
 // Causal attention of every token over its sequence's cache (keys 0..pos, or the last
 // `window` of them), any head_dim that is even and at most 256.
@@ -137,8 +142,9 @@ int rb_fill_normal(void* out, int dtype, long long n, unsigned long long key, do
 // row0 + (r / block) * period + r % block of dst [dst_rows, width].  block = n_rows places the rows
 // one after another from row0 (q, k, v in one matrix); block 16, period 32, row0 0 and 16 interleave
 // gate and up rows in blocks of 16.
-int rb_place_rows(const void* src, int src_dtype, void* dst, int dst_dtype, long long n_rows, long long width,
-                  long long dst_rows, long long row0, long long block, long long period, void* stream);
+// dst_layout 1: dst is fragment-major (see rb_gemm_bf16; dst_rows % 16 == 0, width % 32 == 0).
+int rb_place_rows(const void* src, int src_dtype, void* dst, int dst_dtype, int dst_layout, long long n_rows,
+                  long long width, long long dst_rows, long long row0, long long block, long long period, void* stream);
 
 // What the GPU reaches, measured the simplest way: rb_probe_read reads `bytes` bytes (a multiple of
 // 16) once with 16-byte loads from `blocks` workgroups of 256 lanes; rb_probe_mfma runs 4 * iters bfloat16 32x32x16 MFMAs in each of `waves`

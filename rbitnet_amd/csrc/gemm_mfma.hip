@@ -33,9 +33,16 @@ static int launch_few_tokens(const GemmTokens& x, const bf16_t* w, void* c, int 
   return gemm_skinny_launch(x, w, c, dtype_out, after, m, n, k, s);
 }
 
-extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out, int epilogue, int m, int n,
-                            int k, float* workspace, void* stream) {
+// fragment-major W (w_layout 1) is for K % 64 == 0 and N % 16 == 0
+static bool layout_ok(int w_layout, int n, int k) {
+  return w_layout == 0 || (w_layout == 1 && k % 64 == 0 && n % 16 == 0);
+}
+
+extern "C" int rb_gemm_bf16(const void* a, const void* w, int w_layout, void* c, int dtype_out, int epilogue, int m,
+                            int n, int k, float* workspace, void* stream) {
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_bf16: bad sizes M=%d N=%d K=%d", m, n, k);
+  RB_REQUIRE(layout_ok(w_layout, n, k), "rb_gemm_bf16: W layout %d with N=%d K=%d (fragment-major needs N %% 16 == 0, K %% 64 == 0)",
+             w_layout, n, k);
   RB_REQUIRE(k % 8 == 0, "rb_gemm_bf16: K=%d must be a multiple of 8 (use rb_gemm_generic)", k);
   RB_REQUIRE(epilogue == 0 || epilogue == 1, "rb_gemm_bf16: unknown epilogue %d", epilogue);
   RB_REQUIRE(epilogue == 0 || n % 32 == 0, "rb_gemm_bf16: gated epilogue needs N=%d to be a multiple of 32", n);
@@ -46,10 +53,10 @@ extern "C" int rb_gemm_bf16(const void* a, const void* w, void* c, int dtype_out
   const bf16_t* wa = (const bf16_t*)w;
   int rc = 0;
   if (tiled_parts(m, n, k, epilogue) >= 1) {
-    rc = gemm_tiled_launch(xa, wa, c, workspace, dtype_out, epilogue, m, n, k, s);
+    rc = gemm_tiled_launch(xa, wa, w_layout == 1, c, workspace, dtype_out, epilogue, m, n, k, s);
   } else {
     const GemmTokens x = {xa, nullptr, 0.f, nullptr};
-    const GemmAfter after = {epilogue, nullptr, nullptr, nullptr};
+    const GemmAfter after = {epilogue, nullptr, nullptr, nullptr, w_layout == 1};
     rc = launch_few_tokens(x, wa, c, dtype_out, after, m, n, k, s);
   }
   if (rc) return rc;
@@ -64,10 +71,12 @@ extern "C" int rb_gemm_bf16_terms_count(int m, int n, int k) {
   return p > 1 ? p : 1;
 }
 
-extern "C" int rb_gemm_bf16_terms(const void* a, const void* w, float* terms, int m, int n, int k, void* stream) {
+extern "C" int rb_gemm_bf16_terms(const void* a, const void* w, int w_layout, float* terms, int m, int n, int k,
+                                  void* stream) {
   const int p = rb_gemm_bf16_terms_count(m, n, k);
-  if (p == 1) return rb_gemm_bf16(a, w, terms, RB_F32, 0, m, n, k, nullptr, stream);
-  const int rc = gemm_tiled_launch((const bf16_t*)a, (const bf16_t*)w, nullptr, terms, RB_F32, 0, m, n, k,
+  if (p == 1) return rb_gemm_bf16(a, w, w_layout, terms, RB_F32, 0, m, n, k, nullptr, stream);
+  RB_REQUIRE(layout_ok(w_layout, n, k), "rb_gemm_bf16_terms: W layout %d with N=%d K=%d", w_layout, n, k);
+  const int rc = gemm_tiled_launch((const bf16_t*)a, (const bf16_t*)w, w_layout == 1, nullptr, terms, RB_F32, 0, m, n, k,
                                    (hipStream_t)stream);
   if (rc) return rc;
   RB_LAUNCH_CHECK();
@@ -79,8 +88,9 @@ extern "C" int rb_gemm_bf16_few_ok(int m, int n, int k) {
 }
 
 extern "C" int rb_gemm_bf16_few(const void* a, const float* squares_in, float eps, const int32_t* rows, const void* w,
-                                void* c, int dtype_out, int epilogue, const float* gain, void* gained,
+                                int w_layout, void* c, int dtype_out, int epilogue, const float* gain, void* gained,
                                 float* squares_out, int m, int n, int k, void* stream) {
+  RB_REQUIRE(layout_ok(w_layout, n, k), "rb_gemm_bf16_few: W layout %d with N=%d K=%d", w_layout, n, k);
   RB_REQUIRE(rb_gemm_bf16_few_ok(m, n, k), "rb_gemm_bf16_few: M=%d N=%d K=%d is not for it (1..16 tokens, K %% 8 == 0)",
              m, n, k);
   RB_REQUIRE(epilogue >= 0 && epilogue <= 3, "rb_gemm_bf16_few: unknown epilogue %d", epilogue);
@@ -91,7 +101,7 @@ extern "C" int rb_gemm_bf16_few(const void* a, const float* squares_in, float ep
   RB_REQUIRE(epilogue != 3 || (gain && gained && squares_out),
              "rb_gemm_bf16_few: epilogue 3 needs the gain and room for the prepared rows");
   const GemmTokens x = {(const bf16_t*)a, squares_in, eps, rows};
-  const GemmAfter after = {epilogue, gain, (bf16_t*)gained, squares_out};
+  const GemmAfter after = {epilogue, gain, (bf16_t*)gained, squares_out, w_layout == 1};
   const int rc = launch_few_tokens(x, (const bf16_t*)w, c, dtype_out, after, m, n, k, (hipStream_t)stream);
   if (rc) return rc;
   RB_LAUNCH_CHECK();

@@ -30,6 +30,7 @@ struct FoldArgs {
   const float* gain;            // epilogue 3: [N]
   bf16_t* gained;               // epilogue 3: [M, N]
   float* squares_out;           // epilogue 3: [M, ceil(N / 16)]
+  int w_frag;                   // W is stored fragment-major (see gemm_internal.h)
 };
 
 // What a lane does with its 4 consecutive sums of token mm, columns nn.. (epilogues 0, 2, 3).
@@ -115,13 +116,19 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
 #pragma unroll
     for (int cb = 0; cb < MB; ++cb) acc[rt][cb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
+  // Where a lane finds its 8 values at depth kstart (a multiple of 32) + 8 kq of row tile rt:
+  // wrow[rt] + kstart * wk.  Rows [N, K]: the row's start + 8 kq, wk = 1.  Fragment-major: the
+  // tile's start + 8 lane, wk = 16 (a block of 16 rows x 32 depth values is 512 values).
+  const bool wf = fa.w_frag != 0;
+  const int wk = wf ? 16 : 1;
   const bf16_t* wrow[R];
   bool wok[R];
 #pragma unroll
   for (int rt = 0; rt < R; ++rt) {
     const int row = n0 + 16 * rt + r;
     wok[rt] = row < n;
-    wrow[rt] = w + (size_t)(wok[rt] ? row : 0) * k;
+    if (wf) wrow[rt] = w + (size_t)(n0 + 16 * rt < n ? n0 + 16 * rt : 0) * k + 8 * lane;
+    else wrow[rt] = w + (size_t)(wok[rt] ? row : 0) * k + 8 * kq;
   }
   const bf16_t* xrow[MB];
   bool xok[MB];
@@ -184,14 +191,23 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
     k_begin = 128 * (wave * base + (wave < extra ? wave : extra));
     Frag8 a[U][R][4], b[U][MB][4];
     auto load_stage = [&](int u, int st) {
-      const int kk = k_begin + 128 * st + 8 * kq;
+      const int ks = k_begin + 128 * st;
+      const int kk = ks + 8 * kq;
+      if (wf) {           // read once, whole lines at a time: past the caches
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int rt = 0; rt < R; ++rt) a[u][rt][j].u = load16(wrow[rt] + kk + 32 * j);
+          for (int rt = 0; rt < R; ++rt) a[u][rt][j].u = load16_stream(wrow[rt] + (size_t)(ks + 32 * j) * 16);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int rt = 0; rt < R; ++rt) a[u][rt][j].u = load16(wrow[rt] + ks + 32 * j);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int cb = 0; cb < MB; ++cb) b[u][cb][j].u = load16(xrow[cb] + kk + 32 * j);
-      }
     };
     auto multiply_stage = [&](int u) {
 #pragma unroll
@@ -230,7 +246,8 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
         const int kk = k0 + 32 * j + 8 * kq;
         const bool in = kk < k_end;
 #pragma unroll
-        for (int rt = 0; rt < R; ++rt) a[rt][j].u = (in && wok[rt]) ? load16(wrow[rt] + kk) : zero16();
+        for (int rt = 0; rt < R; ++rt)
+          a[rt][j].u = (in && wok[rt]) ? load16(wrow[rt] + (size_t)(k0 + 32 * j) * wk) : zero16();
 #pragma unroll
         for (int cb = 0; cb < MB; ++cb) b[cb][j].u = (in && xok[cb]) ? load16(xrow[cb] + kk) : zero16();
       }
@@ -330,7 +347,7 @@ extern "C" void rb_tune(int u, int r, int waves) {       // experiments only; 0 
 }
 
 static FoldArgs fold_args(const GemmTokens& x, const GemmAfter& after) {
-  return FoldArgs{x.squares, x.rows, x.eps, after.gain, after.gained, after.squares};
+  return FoldArgs{x.squares, x.rows, x.eps, after.gain, after.gained, after.squares, after.w_frag ? 1 : 0};
 }
 
 template <int MB, int R, int U, bool FAST, int EPI, typename TO, bool SCALED>
@@ -444,6 +461,15 @@ __global__ __launch_bounds__(512) void gemm_resident_kernel(const bf16_t* __rest
   if (t_count <= 0) return;
   Frag8 a0[XQ], a1[XQ];
   auto load_tile = [&](Frag8* a, int t) {
+    if (fa.w_frag) {
+      // fragment-major: the wave's XQ blocks of a tile are XQ KB in a row; read once, past the caches
+      int tile = tile0 + t;
+      if (tile * 16 >= n) tile = 0;              // results of such rows are never stored
+      const bf16_t* p = w + ((size_t)tile * k + (size_t)(blockIdx.y * n_waves + wave) * (32 * XQ)) * 16 + 8 * lane;
+#pragma unroll
+      for (int j = 0; j < XQ; ++j) a[j].u = load16_stream(p + (size_t)j * 512);
+      return;
+    }
     int row = (tile0 + t) * 16 + r;
     if (row >= n) row = 0;                       // results of such rows are never stored
     const bf16_t* wrow = w + (size_t)row * k + k0;

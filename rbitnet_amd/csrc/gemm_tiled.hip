@@ -251,7 +251,7 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_tiled_kernel(
 // The loads are inline assembly, so the compiler neither counts nor waits for them: the
 // kernel waits itself (s_waitcnt vmcnt) for the stage it is about to read, leaving the
 // younger stages in flight.  There is no other memory access in the main loop.
-template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO>
+template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO, bool WF>
 __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(const bf16_t* __restrict__ x,
                                                        const bf16_t* __restrict__ w, TO* __restrict__ c,
                                                        float* __restrict__ slabs, int m, int n, int k, int m_tiles,
@@ -298,11 +298,21 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   uint32_t woff[W_LOADS], xoff[X_LOADS];        // byte offsets from the tile's first element, without the k-tile
 #pragma unroll
   for (int i = 0; i < W_LOADS; ++i) {
-    const int row = (wave + NWAVES * i) * RPW + lane / CPR;
-    const int chunk = (lane % CPR) ^ ((row / RPB) % CPR);
-    int grow = row;
-    if (n0 + grow > n - 1) grow = n - 1 - n0;   // rows beyond N: any valid row, never stored
-    woff[i] = ((uint32_t)grow * (uint32_t)k + chunk * 8) * 2u;
+    if (WF) {
+      // W fragment-major: wave-wide load q fetches one block of 16 rows x 32 depth values, 1 KB in
+      // a row, and the stage holds the tile's blocks in the order [BN / 16][BK / 32]
+      const int q = wave + NWAVES * i;
+      int rt = q / (BK / 32);
+      const int kb = q % (BK / 32);
+      if (n0 + 16 * rt >= n) rt = 0;            // rows beyond N: any valid tile, never stored
+      woff[i] = ((uint32_t)(16 * rt) * (uint32_t)k + (uint32_t)kb * 512u + (uint32_t)lane * 8u) * 2u;
+    } else {
+      const int row = (wave + NWAVES * i) * RPW + lane / CPR;
+      const int chunk = (lane % CPR) ^ ((row / RPB) % CPR);
+      int grow = row;
+      if (n0 + grow > n - 1) grow = n - 1 - n0;   // rows beyond N: any valid row, never stored
+      woff[i] = ((uint32_t)grow * (uint32_t)k + chunk * 8) * 2u;
+    }
   }
 #pragma unroll
   for (int i = 0; i < X_LOADS; ++i) {
@@ -314,12 +324,14 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;      // LDS byte address of stage 0
   const int kt0 = blockIdx.y * k_tiles;                    // this workgroup's slice of K: k_tiles tiles from here
+  // a K tile further on: BK values along a row, or BK / 32 blocks of 1 KB (fragment-major)
+  constexpr uint32_t W_KSTEP = WF ? BK * 32 : BK * 2;
   auto issue = [&](int kt) {
     const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
     const uint32_t kbytes = (uint32_t)(kt0 + kt) * (BK * 2);
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i)
-      load_to_lds16(wtile, woff[i] + kbytes, stage + (uint32_t)(wave + NWAVES * i) * 1024u);
+      load_to_lds16(wtile, woff[i] + (uint32_t)(kt0 + kt) * W_KSTEP, stage + (uint32_t)(wave + NWAVES * i) * 1024u);
 #pragma unroll
     for (int i = 0; i < X_LOADS; ++i)
       load_to_lds16(xtile, xoff[i] + kbytes, stage + (uint32_t)(BN * BK * 2) + (uint32_t)(wave + NWAVES * i) * 1024u);
@@ -329,15 +341,22 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   constexpr int KSTEPS = BK / 16;
   static_assert(KSTEPS % 2 == 0, "the fragment buffers alternate by depth step");
   const int sw = (l32 / RPB) % CPR;
-  const bf16_t* wfrag = lds + (size_t)(wn0 + l32) * BK;
+  // W's fragments.  Rows: row wn0 + 32 i + l32, chunk 2 ks + g in slot chunk ^ sw.  Fragment-major:
+  // block [(wn0 + 32 i + l32) / 16][chunk / 4], inside it 16 bytes at 16 ((chunk % 4) * 16 + l32 % 16);
+  // the 16 lanes that are served together read 256 bytes in a row.
+  const bf16_t* wfrag = WF ? lds + ((size_t)((wn0 + l32) / 16) * (BK / 32) * 64 + (l32 % 16)) * 8
+                           : lds + (size_t)(wn0 + l32) * BK;
+  constexpr int W_ISTEP = WF ? 2 * (BK / 32) * 512 : 32 * BK;       // 32 rows further on
+  auto w_slot = [&](int ks) { return WF ? (((2 * ks + g) / 4) * 64 + ((2 * ks + g) % 4) * 16) * 8 : ((2 * ks + g) ^ sw) * 8; };
   const bf16_t* xfrag = lds + (size_t)BN * BK + (size_t)(wm0 + l32) * BK;
   Frag8 a[2][TN], b[2][TM];
   auto load_frags = [&](int buf2, int kt, int ks) {
     const bf16_t* wb = wfrag + (size_t)(kt % S) * STAGE;
     const bf16_t* xb = xfrag + (size_t)(kt % S) * STAGE;
     const int slot = ((2 * ks + g) ^ sw) * 8;
+    const int wslot = w_slot(ks);
 #pragma unroll
-    for (int i = 0; i < TN; ++i) a[buf2][i].u = *reinterpret_cast<const uint4*>(wb + 32 * i * BK + slot);
+    for (int i = 0; i < TN; ++i) a[buf2][i].u = *reinterpret_cast<const uint4*>(wb + i * W_ISTEP + wslot);
 #pragma unroll
     for (int j = 0; j < TM; ++j) b[buf2][j].u = *reinterpret_cast<const uint4*>(xb + 32 * j * BK + slot);
   };
@@ -365,7 +384,8 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   auto issue_one = [&](int kt, int l) {
     const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
     const uint32_t kbytes = (uint32_t)(kt0 + kt) * (BK * 2);
-    if (l < W_LOADS) load_to_lds16(wtile, woff[l] + kbytes, stage + (uint32_t)(wave + NWAVES * l) * 1024u);
+    if (l < W_LOADS)
+      load_to_lds16(wtile, woff[l] + (uint32_t)(kt0 + kt) * W_KSTEP, stage + (uint32_t)(wave + NWAVES * l) * 1024u);
     else
       load_to_lds16(xtile, xoff[l - W_LOADS] + kbytes,
                     stage + (uint32_t)(BN * BK * 2) + (uint32_t)(wave + NWAVES * (l - W_LOADS)) * 1024u);
@@ -376,7 +396,7 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
     const int slot = ((2 * ks + g) ^ sw) * 8;
     if (f == 0 || f > TM) {
       const int i = f == 0 ? 0 : f - TM;
-      a[buf2][i].u = *reinterpret_cast<const uint4*>(wfrag + (size_t)(kt % S) * STAGE + 32 * i * BK + slot);
+      a[buf2][i].u = *reinterpret_cast<const uint4*>(wfrag + (size_t)(kt % S) * STAGE + i * W_ISTEP + w_slot(ks));
     } else {
       b[buf2][f - 1].u = *reinterpret_cast<const uint4*>(xfrag + (size_t)(kt % S) * STAGE + 32 * (f - 1) * BK + slot);
     }
@@ -491,7 +511,7 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
       store_piece<EPI, TO>(acc[i][j], c, slab, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n);
 }
 
-template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO>
+template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO, bool WF>
 static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s,
                           int parts = 1, float* slabs = nullptr) {
   const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
@@ -503,7 +523,8 @@ static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int 
   // byte offsets inside a tile are 32-bit
   RB_REQUIRE((long long)(BN > BM ? BN : BM) * k * 2 < (1LL << 32), "rb_gemm_bf16: K=%d too long for this kernel", k);
   const size_t lds = (size_t)S * (BN + BM) * BK * sizeof(bf16_t);
-  auto kern = gemm_dma_kernel<BN, BM, WN, WM, BK, S, EPI, TO>;
+  RB_REQUIRE(!WF || (BN % 32 == 0 && n % 16 == 0), "rb_gemm_bf16: fragment-major W needs N=%d to be a multiple of 16", n);
+  auto kern = gemm_dma_kernel<BN, BM, WN, WM, BK, S, EPI, TO, WF>;
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -647,7 +668,7 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   return {7, epilogue ? 1 : k_slices(t64, k, 256, k / (8 * m))};
 }
 
-template <int EPI, typename TO>
+template <int EPI, typename TO, bool WF>
 static int launch_planned(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int m, int n, int k,
                           hipStream_t s) {
   const TilePlan plan = plan_tiles(m, n, k, EPI);
@@ -656,30 +677,38 @@ static int launch_planned(const bf16_t* x, const bf16_t* w, void* c, float* work
              m, n, k, (long long)plan.parts * m * n);
   const int p = plan.parts;
   switch (plan.cfg) {
-    case 8: return launch_dma_cfg<256, 128, 64, 64, 64, 3, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
-    case 9: return launch_dma_cfg<320, 256, 160, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
-    case 7: return launch_dma_cfg<128, 64, 32, 64, 64, 3, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
-    case 10: return launch_dma_cfg<64, 64, 32, 32, 64, 4, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
-    case 13: return launch_dma_cfg<128, 64, 32, 64, 128, 3, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
-    case 6: return launch_dma_cfg<192, 256, 96, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
-    case 5: return launch_dma_cfg<128, 128, 64, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
-    case 4: return launch_dma_cfg<256, 256, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, p, workspace);
-    case 3: return launch_tiled_cfg<256, 256, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
-    case 2: return launch_tiled_cfg<256, 128, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
-    default: return launch_tiled_cfg<128, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+    case 8: return launch_dma_cfg<256, 128, 64, 64, 64, 3, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
+    case 9: return launch_dma_cfg<320, 256, 160, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
+    case 7: return launch_dma_cfg<128, 64, 32, 64, 64, 3, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
+    case 10: return launch_dma_cfg<64, 64, 32, 32, 64, 4, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
+    case 13: return launch_dma_cfg<128, 64, 32, 64, 128, 3, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
+    case 6: return launch_dma_cfg<192, 256, 96, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
+    case 5: return launch_dma_cfg<128, 128, 64, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
+    case 4: return launch_dma_cfg<256, 256, 128, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
+    default: break;
   }
+  if constexpr (!WF) {
+    switch (plan.cfg) {
+      case 3: return launch_tiled_cfg<256, 256, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+      case 2: return launch_tiled_cfg<256, 128, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+      default: return launch_tiled_cfg<128, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+    }
+  }
+  RB_REQUIRE(false, "rb_gemm_bf16: internal: fragment-major W with K=%d, which the direct-to-LDS kernels do not take", k);
+  return 1;
 }
 
-#define RB_BY_OUTPUT(FN, ...)                                                              \
-  (epilogue == 0 ? (dtype_out == RB_F32 ? FN<0, float>(__VA_ARGS__) : FN<0, bf16_t>(__VA_ARGS__)) \
-                 : (dtype_out == RB_F32 ? FN<1, float>(__VA_ARGS__) : FN<1, bf16_t>(__VA_ARGS__)))
+#define RB_BY_OUTPUT(FN, WF, ...)                                                              \
+  (epilogue == 0 ? (dtype_out == RB_F32 ? FN<0, float, WF>(__VA_ARGS__) : FN<0, bf16_t, WF>(__VA_ARGS__)) \
+                 : (dtype_out == RB_F32 ? FN<1, float, WF>(__VA_ARGS__) : FN<1, bf16_t, WF>(__VA_ARGS__)))
 
 int gemm_tiled_parts(int m, int n, int k, int epilogue) {
   const TilePlan plan = plan_tiles(m, n, k, epilogue);
   return plan.cfg == 0 ? 0 : plan.parts;
 }
 
-int gemm_tiled_launch(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int dtype_out, int epilogue, int m,
-                      int n, int k, hipStream_t s) {
-  return RB_BY_OUTPUT(launch_planned, x, w, c, workspace, m, n, k, s);
+int gemm_tiled_launch(const bf16_t* x, const bf16_t* w, bool w_frag, void* c, float* workspace, int dtype_out,
+                      int epilogue, int m, int n, int k, hipStream_t s) {
+  if (w_frag) return RB_BY_OUTPUT(launch_planned, true, x, w, c, workspace, m, n, k, s);
+  return RB_BY_OUTPUT(launch_planned, false, x, w, c, workspace, m, n, k, s);
 }

@@ -129,11 +129,11 @@ class Kernels:
             "rb_rope_kv_write": [_P, _I, ctypes.c_longlong, _P, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
             "rb_swiglu": [_P, _P, _I, _I, _I, _P],
             "rb_gemm_generic": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
-            "rb_gemm_bf16": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P],
-            "rb_gemm_bf16_few": [_P, _P, _F, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _P],
+            "rb_gemm_bf16": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _P, _P],
+            "rb_gemm_bf16_few": [_P, _P, _F, _P, _P, _I, _P, _I, _I, _P, _P, _P, _I, _I, _I, _P],
             "rb_gemm_bf16_few_ok": [_I, _I, _I],
             "rb_gemm_bf16_terms_count": [_I, _I, _I],
-            "rb_gemm_bf16_terms": [_P, _P, _P, _I, _I, _I, _P],
+            "rb_gemm_bf16_terms": [_P, _P, _I, _P, _I, _I, _I, _P],
             "rb_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_prefill_bf16": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
             "rb_attention_decode_bf16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
@@ -141,7 +141,7 @@ class Kernels:
                                                _P, _P],
             "rb_sample": [_P, _I, _I, _P, _P, _P, _P, _P],
             "rb_fill_normal": [_P, _I, ctypes.c_longlong, ctypes.c_ulonglong, ctypes.c_double, ctypes.c_double, _P],
-            "rb_place_rows": [_P, _I, _P, _I] + [ctypes.c_longlong] * 6 + [_P],
+            "rb_place_rows": [_P, _I, _P, _I, _I] + [ctypes.c_longlong] * 6 + [_P],
             "rb_probe_read": [_P, ctypes.c_longlong, _I, _P, _P],
             "rb_probe_mfma": [_I, _I, _P, _P],
         }
@@ -244,7 +244,9 @@ class Kernels:
         self._ok(self._lib.rb_gemm_generic(_ptr(a), _ptr(w), _ptr(c), dtype_code(a.dtype), dtype_code(c.dtype),
                                            m, n, k, self._stream()))
 
-    def gemm_bf16(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = 0) -> None:
+    def gemm_bf16(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = 0,
+                  w_frag: bool = False) -> None:
+        """w_frag: w [N, K] is stored fragment-major (`place_rows(..., frag=True)` writes that)."""
         m, k = a.shape
         n = w.shape[0]
         _check(a, "a", torch.bfloat16)
@@ -252,13 +254,13 @@ class Kernels:
         _check(c, "c", None, (m, n // 2 if epilogue == 1 else n))
         need = int(self._lib.rb_gemm_workspace_floats(m, n, k, int(epilogue)))
         workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need else None
-        self._ok(self._lib.rb_gemm_bf16(_ptr(a), _ptr(w), _ptr(c), dtype_code(c.dtype), int(epilogue), m, n, k,
-                                        _ptr(workspace), self._stream()))
+        self._ok(self._lib.rb_gemm_bf16(_ptr(a), _ptr(w), int(bool(w_frag)), _ptr(c), dtype_code(c.dtype), int(epilogue),
+                                        m, n, k, _ptr(workspace), self._stream()))
 
     def gemm_bf16_terms_count(self, m: int, n: int, k: int) -> int:
         return int(self._lib.rb_gemm_bf16_terms_count(int(m), int(n), int(k)))
 
-    def gemm_bf16_terms(self, a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    def gemm_bf16_terms(self, a: torch.Tensor, w: torch.Tensor, w_frag: bool = False) -> torch.Tensor:
         """a w^T as float32 terms [P, M, N] to be added up in their order: what the K slices of
         the kernel for these sizes computed (P = 1: the product itself)."""
         m, k = a.shape
@@ -267,7 +269,7 @@ class Kernels:
         _check(w, "w", torch.bfloat16, (n, k))
         terms = torch.empty((int(self._lib.rb_gemm_bf16_terms_count(m, n, k)), m, n), dtype=torch.float32,
                             device=a.device)
-        self._ok(self._lib.rb_gemm_bf16_terms(_ptr(a), _ptr(w), _ptr(terms), m, n, k, self._stream()))
+        self._ok(self._lib.rb_gemm_bf16_terms(_ptr(a), _ptr(w), int(bool(w_frag)), _ptr(terms), m, n, k, self._stream()))
         return terms
 
     def gemm_bf16_few_ok(self, m: int, n: int, k: int) -> bool:
@@ -277,7 +279,7 @@ class Kernels:
     def gemm_bf16_few(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = 0,
                       squares: Optional[torch.Tensor] = None, eps: float = 0.0, rows: Optional[torch.Tensor] = None,
                       gain: Optional[torch.Tensor] = None, gained: Optional[torch.Tensor] = None,
-                      squares_out: Optional[torch.Tensor] = None) -> None:
+                      squares_out: Optional[torch.Tensor] = None, w_frag: bool = False) -> None:
         """The product of 1..16 tokens with its neighbours folded in.
         squares [*, ceil(K / 16)]: a holds rows times a norm's gain and squares the sums of squares
         of the rows themselves; the product is scaled to that of the RMS-normalised rows (eps).
@@ -299,8 +301,8 @@ class Kernels:
             _check(gain, "gain", torch.float32, (n,))
             _check(gained, "gained", torch.bfloat16, (m, n))
             _check(squares_out, "squares_out", torch.float32, (m, (n + 15) // 16))
-        self._ok(self._lib.rb_gemm_bf16_few(_ptr(a), _ptr(squares), float(eps), _ptr(rows), _ptr(w), _ptr(c),
-                                            dtype_code(c.dtype), int(epilogue), _ptr(gain), _ptr(gained),
+        self._ok(self._lib.rb_gemm_bf16_few(_ptr(a), _ptr(squares), float(eps), _ptr(rows), _ptr(w), int(bool(w_frag)),
+                                            _ptr(c), dtype_code(c.dtype), int(epilogue), _ptr(gain), _ptr(gained),
                                             _ptr(squares_out), m, n, k, self._stream()))
 
     def attention_generic(self, q, k_pages, v_pages, out, tok_pos, tok_seq, block_table, n_heads, n_kv, head_dim,
@@ -405,9 +407,10 @@ class Kernels:
                                           float(mean), float(std), self._stream()))
 
     def place_rows(self, src: torch.Tensor, dst: torch.Tensor, row0: int = 0, block: Optional[int] = None,
-                   period: Optional[int] = None) -> None:
+                   period: Optional[int] = None, frag: bool = False) -> None:
         """Row r of src goes, cast to dst's dtype, to row row0 + (r // block) * period + r % block
-        of dst (block: all rows, so that they follow one another from row0)."""
+        of dst (block: all rows, so that they follow one another from row0).  frag: dst is stored
+        fragment-major (the matrix-core products' other layout of W; rows % 16 == 0, width % 32 == 0)."""
         _check(src, "src")
         _check(dst, "dst")
         if src.dim() != 2 or dst.dim() != 2 or src.shape[1] != dst.shape[1]:
@@ -415,8 +418,9 @@ class Kernels:
         n = src.shape[0]
         block = max(1, n) if block is None else int(block)
         period = block if period is None else int(period)
-        self._ok(self._lib.rb_place_rows(_ptr(src), dtype_code(src.dtype), _ptr(dst), dtype_code(dst.dtype), n,
-                                         src.shape[1], dst.shape[0], int(row0), block, period, self._stream()))
+        self._ok(self._lib.rb_place_rows(_ptr(src), dtype_code(src.dtype), _ptr(dst), dtype_code(dst.dtype),
+                                         int(bool(frag)), n, src.shape[1], dst.shape[0], int(row0), block, period,
+                                         self._stream()))
 
     # ------------------------------------------------------------------ probes
     def probe_read(self, buf: torch.Tensor, sink: torch.Tensor, blocks: int = 2048) -> None:

@@ -121,13 +121,17 @@ __global__ __launch_bounds__(256) void fill_normal_kernel(T* __restrict__ out, l
 template <typename S, typename T>
 __global__ __launch_bounds__(256) void place_rows_kernel(const S* __restrict__ src, T* __restrict__ dst,
                                                          long long n_rows, long long width, long long row0,
-                                                         long long block, long long period) {
+                                                         long long block, long long period, int frag) {
   const long long total = n_rows * width;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (long long)gridDim.x * blockDim.x) {
     const long long r = i / width, c = i - r * width;
     const long long d = row0 + (r / block) * period + r % block;
-    Num<T>::store(dst + d * width + c, Num<S>::load(src + i));
+    // fragment-major: blocks of 16 rows x 32 columns in the order [rows / 16][width / 32]; inside a
+    // block the value of row r, column q lies at 8 * (16 * (q / 8) + r) + q % 8
+    const long long at = frag ? ((d / 16) * (width / 32) + c / 32) * 512 + (16 * ((c % 32) / 8) + d % 16) * 8 + c % 8
+                              : d * width + c;
+    Num<T>::store(dst + at, Num<S>::load(src + i));
   }
 }
 
@@ -154,9 +158,11 @@ extern "C" int rb_fill_normal(void* out, int dtype, long long n, unsigned long l
   return 0;
 }
 
-extern "C" int rb_place_rows(const void* src, int src_dtype, void* dst, int dst_dtype, long long n_rows,
-                             long long width, long long dst_rows, long long row0, long long block, long long period,
-                             void* stream) {
+extern "C" int rb_place_rows(const void* src, int src_dtype, void* dst, int dst_dtype, int dst_layout,
+                             long long n_rows, long long width, long long dst_rows, long long row0, long long block,
+                             long long period, void* stream) {
+  RB_REQUIRE(dst_layout == 0 || (dst_layout == 1 && dst_rows % 16 == 0 && width % 32 == 0),
+             "rb_place_rows: layout %d of a destination of %lld rows of %lld", dst_layout, dst_rows, width);
   RB_REQUIRE(n_rows >= 0 && width > 0 && block > 0 && period >= block && row0 >= 0,
              "rb_place_rows: bad sizes (rows %lld, width %lld, block %lld, period %lld, first row %lld)", n_rows, width,
              block, period, row0);
@@ -168,7 +174,7 @@ extern "C" int rb_place_rows(const void* src, int src_dtype, void* dst, int dst_
   hipStream_t s = (hipStream_t)stream;
   const int grid = grid_for(n_rows * width);
 #define RB_PLACE(S, T) \
-  place_rows_kernel<S, T><<<grid, 256, 0, s>>>((const S*)src, (T*)dst, n_rows, width, row0, block, period)
+  place_rows_kernel<S, T><<<grid, 256, 0, s>>>((const S*)src, (T*)dst, n_rows, width, row0, block, period, dst_layout)
   if (src_dtype == RB_F32 && dst_dtype == RB_F32)
     RB_PLACE(float, float);
   else if (src_dtype == RB_F32)

@@ -17,7 +17,7 @@ from ..config.spec import ModelSpec
 from ..errors import ConfigError
 from ..parts.base import BuildEnv, CacheRequest, TensorSpec, build_part
 from ..parts.block import normed_for
-from ..parts.linear import linear
+from ..parts.linear import linear, pack_rows
 
 
 def _build_blocks(spec: ModelSpec, env_for: Callable[[int], BuildEnv]):
@@ -74,6 +74,7 @@ class Model:
         self.dtype = dtype
         self.device = torch.device(device)
         self.lib = lib
+        self.generic_only = generic_only
 
         shared: Dict = {}
 
@@ -152,7 +153,12 @@ class Model:
         spec = self.spec
         placed = lambda name: self._place(tensors[name], self.expected[name])
         self.embedding = placed(spec.embedding_name)
-        self.head = self.embedding if spec.head_name is None else placed(spec.head_name)
+        if spec.head_name is None:
+            self.head = self.embedding            # tied: the table's rows are also read one by one
+        else:
+            head = placed(spec.head_name)
+            self.head = pack_rows(self.lib, [(head, 0, None, None)], head.shape[0], head.shape[1], head.dtype,
+                                  head.device, not self.generic_only)
         for prefix, part in _named_parts(spec, self.blocks, self.final_norm).items():
             part.load({name: placed(f"{prefix}.{name}") for name in part.tensor_specs()})
         norm_specs = self.final_norm.tensor_specs()

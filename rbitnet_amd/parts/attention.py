@@ -32,7 +32,7 @@ import torch
 
 from ..errors import ConfigError
 from .base import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register_mixer
-from .linear import linear, linear_or_terms, linear_to_stream
+from .linear import linear, linear_or_terms, linear_to_stream, pack_rows
 
 DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight"}
 _MATRIX_CORE_HEAD_DIMS = (64, 128)
@@ -76,17 +76,17 @@ class Attention(Part):
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         # q, k and v rows in one matrix: one product per step instead of three
-        if self.cache_from is None:
-            parts = [tensors[self.names[n]] for n in ("q", "k", "v")]
-            self.w_qkv = torch.empty((sum(p.shape[0] for p in parts), self.hidden), dtype=parts[0].dtype,
-                                     device=parts[0].device)
-            row = 0
-            for p in parts:
-                self.env.lib.place_rows(p.contiguous(), self.w_qkv, row0=row)
-                row += p.shape[0]
-        else:
-            self.w_qkv = tensors[self.names["q"]].contiguous()
-        self.w_o = tensors[self.names["o"]].contiguous()
+        lib, allowed = self.env.lib, not getattr(self.env, "generic_only", False)
+        names = ("q", "k", "v") if self.cache_from is None else ("q",)
+        pieces, row = [], 0
+        for n in names:
+            t = tensors[self.names[n]]
+            pieces.append((t, row, None, None))
+            row += t.shape[0]
+        first = pieces[0][0]
+        self.w_qkv = pack_rows(lib, pieces, row, self.hidden, first.dtype, first.device, allowed)
+        o = tensors[self.names["o"]]
+        self.w_o = pack_rows(lib, [(o, 0, None, None)], o.shape[0], o.shape[1], o.dtype, o.device, allowed)
 
     def cache_request(self) -> Optional[CacheRequest]:
         if self.cache_from is not None:

@@ -18,7 +18,7 @@ import torch
 
 from ..errors import ConfigError
 from .base import BuildEnv, Part, TensorSpec, register_feed_forward
-from .linear import can_fuse_gate, gated_linear, linear_to_stream, pack_gate_up
+from .linear import can_fuse_gate, gated_linear, linear_to_stream, pack_gate_up, pack_rows
 
 DEFAULT_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
 
@@ -45,8 +45,12 @@ class SwiGLU(Part):
                 self.names["down"]: TensorSpec((self.hidden, self.ff))}
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.w_gate_up = pack_gate_up(self.env.lib, tensors[self.names["gate"]], tensors[self.names["up"]], self.fused)
-        self.w_down = tensors[self.names["down"]].contiguous()
+        allowed = not getattr(self.env, "generic_only", False)
+        self.w_gate_up = pack_gate_up(self.env.lib, tensors[self.names["gate"]], tensors[self.names["up"]], self.fused,
+                                      allowed)
+        down = tensors[self.names["down"]]
+        self.w_down = pack_rows(self.env.lib, [(down, 0, None, None)], down.shape[0], down.shape[1], down.dtype,
+                                down.device, allowed)
 
     def forward(self, h, ctx=None, stream: Optional[torch.Tensor] = None, next_norm=None):
         lib = self.env.lib

@@ -130,3 +130,11 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor, block: int = 16) ->
     g = gate.reshape(ff // block, block, k)
     u = up.reshape(ff // block, block, k)
     return torch.stack([g, u], dim=1).reshape(2 * ff, k).contiguous()
+
+
+def fragment_major(w: torch.Tensor) -> torch.Tensor:
+    """[N, K] (N % 16 == 0, K % 32 == 0) in the matrix-core products' other layout of W: blocks of
+    16 rows x 32 columns in the order [N / 16][K / 32]; inside a block the value of row r, column q
+    at 8 * (16 * (q / 8) + r) + q % 8.  Built with torch, as the oracle of the packing kernel."""
+    n, k = w.shape
+    return w.reshape(n // 16, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(n, k)

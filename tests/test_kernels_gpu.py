@@ -758,3 +758,54 @@ def test_probes_run(lib):
     assert torch.equal(buf, before) and float(sink) == 0.0
     with pytest.raises(KernelError):
         lib.probe_read(buf[:3], sink)
+
+
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 40, 64, 100, 256, 700, 2100])
+@pytest.mark.parametrize("n,k,epi", [(4096, 1024, 0), (1008, 64, 0), (48, 128, 0), (6144, 4096, 0), (12288, 448, 0),
+                                     (672, 256, 1), (8208 * 2, 384, 1), (28672, 512, 1)])
+def test_gemm_bf16_with_w_stored_fragment_major(lib, m, n, k, epi):
+    """Every matrix-core product kernel (tokens in registers, W streamed; tiles through LDS, with and
+    without K slices) reads W in either layout and gives the same numbers bit for bit: the layout
+    changes where a value lies, not which values a sum adds in which order."""
+    from helpers import fragment_major
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(n, k, generator=g) * 0.3).bfloat16()
+    rows, frag = w.to(DEV), fragment_major(w).to(DEV)
+    # the packing kernel writes the same layout
+    packed = torch.full((n, k), float("nan"), dtype=torch.bfloat16, device=DEV)
+    lib.place_rows(rows, packed, frag=True)
+    assert torch.equal(packed, frag)
+    shape = (m, n // 2 if epi else n)
+    for dtype in (torch.float32, torch.bfloat16):
+        want = torch.full(shape, float("nan"), device=DEV, dtype=dtype)
+        got = torch.full(shape, float("nan"), device=DEV, dtype=dtype)
+        lib.gemm_bf16(a, rows, want, epi)
+        lib.gemm_bf16(a, frag, got, epi, w_frag=True)
+        assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
+    if not epi:
+        assert torch.equal(lib.gemm_bf16_terms(a, frag, w_frag=True), lib.gemm_bf16_terms(a, rows))
+        oracle = a.double().cpu() @ w.double().T
+        assert _rel(want.float(), oracle) < 1e-2
+    if m <= 16 and not epi and lib.gemm_bf16_few_ok(m, n, k):
+        for epilogue in (2, 3):
+            outs = []
+            for mat, is_frag in ((rows, False), (frag, True)):
+                c = torch.ones((m, n), device=DEV)
+                gain = torch.linspace(0.5, 1.5, n, device=DEV)
+                gained = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+                squares = torch.empty((m, (n + 15) // 16), device=DEV)
+                lib.gemm_bf16_few(a, mat, c, epilogue, gain=gain, gained=gained, squares_out=squares, w_frag=is_frag)
+                outs.append((c, gained, squares) if epilogue == 3 else (c,))
+            for x, y in zip(*outs):
+                assert torch.equal(x, y)
+
+
+def test_fragment_major_refuses_sizes_it_is_not_for(lib):
+    from rbitnet_amd.errors import KernelError
+    a = torch.zeros(4, 72, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(32, 72, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelError, match="fragment-major"):
+        lib.gemm_bf16(a, w, torch.empty(4, 32, device=DEV), 0, w_frag=True)
+    with pytest.raises(KernelError, match="layout"):
+        lib.place_rows(torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV), frag=True)
