@@ -326,12 +326,23 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   const int kt0 = blockIdx.y * k_tiles;                    // this workgroup's slice of K: k_tiles tiles from here
   // a K tile further on: BK values along a row, or BK / 32 blocks of 1 KB (fragment-major)
   constexpr uint32_t W_KSTEP = WF ? BK * 32 : BK * 2;
+  // With one tile of tokens every workgroup reads rows of W that nobody else reads, once: whole
+  // lines (fragment-major) past the caches, as the products of few tokens do.  Only where a
+  // workgroup's walk along K is long: the short walks of a product cut into many K slices are
+  // bound by their first loads, which come sooner through the caches (64 tokens: 28,672 gated rows
+  // 51 -> 43 us with such loads, but 4,096 rows in 8 slices of 8 tiles 15 -> 16.6 us).
+  const bool w_once = WF && m_tiles == 1 && k_tiles >= 24;
   auto issue = [&](int kt) {
     const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
     const uint32_t kbytes = (uint32_t)(kt0 + kt) * (BK * 2);
 #pragma unroll
-    for (int i = 0; i < W_LOADS; ++i)
-      load_to_lds16(wtile, woff[i] + (uint32_t)(kt0 + kt) * W_KSTEP, stage + (uint32_t)(wave + NWAVES * i) * 1024u);
+    for (int i = 0; i < W_LOADS; ++i) {
+      if (w_once)
+        load_to_lds16_stream(wtile, woff[i] + (uint32_t)(kt0 + kt) * W_KSTEP,
+                             stage + (uint32_t)(wave + NWAVES * i) * 1024u);
+      else
+        load_to_lds16(wtile, woff[i] + (uint32_t)(kt0 + kt) * W_KSTEP, stage + (uint32_t)(wave + NWAVES * i) * 1024u);
+    }
 #pragma unroll
     for (int i = 0; i < X_LOADS; ++i)
       load_to_lds16(xtile, xoff[i] + kbytes, stage + (uint32_t)(BN * BK * 2) + (uint32_t)(wave + NWAVES * i) * 1024u);
@@ -384,8 +395,13 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   auto issue_one = [&](int kt, int l) {
     const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
     const uint32_t kbytes = (uint32_t)(kt0 + kt) * (BK * 2);
-    if (l < W_LOADS)
-      load_to_lds16(wtile, woff[l] + (uint32_t)(kt0 + kt) * W_KSTEP, stage + (uint32_t)(wave + NWAVES * l) * 1024u);
+    if (l < W_LOADS) {
+      if (w_once)
+        load_to_lds16_stream(wtile, woff[l] + (uint32_t)(kt0 + kt) * W_KSTEP,
+                             stage + (uint32_t)(wave + NWAVES * l) * 1024u);
+      else
+        load_to_lds16(wtile, woff[l] + (uint32_t)(kt0 + kt) * W_KSTEP, stage + (uint32_t)(wave + NWAVES * l) * 1024u);
+    }
     else
       load_to_lds16(xtile, xoff[l - W_LOADS] + kbytes,
                     stage + (uint32_t)(BN * BK * 2) + (uint32_t)(wave + NWAVES * (l - W_LOADS)) * 1024u);

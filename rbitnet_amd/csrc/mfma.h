@@ -57,6 +57,18 @@ __device__ __forceinline__ float silu_f32(float v) {
 template <int N>
 __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
+// the same for data that is read once and by nobody else: past the caches
+__device__ __forceinline__ void load_to_lds16_stream(const bf16_t* base, uint32_t byte_offset,
+                                                     uint32_t lds_byte_address) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2 nt"
+      :
+      : "s"(lds_byte_address), "v"(byte_offset), "s"(base)
+      : "memory");
+}
+
 __device__ __forceinline__ void load_to_lds16(const bf16_t* base, uint32_t byte_offset, uint32_t lds_byte_address) {
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
