@@ -99,7 +99,9 @@ def decode_run(engine, batch: int, steps: int, warmup: int, seed: int = 0, promp
 
 
 def probe(lib, device) -> dict:
-    """What this GPU reaches on a plain streaming read and on back-to-back bfloat16 MFMAs
+    """What this GPU reaches on a streaming read (`read_*`: all workgroups striding through the
+    buffer together with plain loads; `stream_*`: every workgroup walking pieces of its own with
+    non-temporal loads, as the decode products read their weights) and on back-to-back bfloat16 MFMAs
     (csrc/probe.hip): the practical ceilings beside the nominal peaks.  Timed with events on
     the stream, so that launch overhead on the host does not count."""
     import torch
@@ -118,12 +120,14 @@ def probe(lib, device) -> dict:
 
     out = {}
     pool = torch.empty((3 << 30) // 4, dtype=torch.int32, device=device).fill_(1)
-    for label, nbytes in (("read_1gb_gbps", 1 << 30), ("read_32mb_gbps", 32 << 20)):
+    for label, nbytes, pieces in (("read_1gb_gbps", 1 << 30, False), ("read_32mb_gbps", 32 << 20, False),
+                                  ("stream_1gb_gbps", 1 << 30, True), ("stream_32mb_gbps", 32 << 20, True)):
         copies = pool.numel() * 4 // nbytes
         views = [pool[i * (nbytes // 4):(i + 1) * (nbytes // 4)] for i in range(copies)]
         best = 0.0
         for blocks in (1024, 2048, 4096, 8192):          # the best grid size counts
-            t = timed(lambda i: lib.probe_read(views[i % copies], sink, blocks), 12 if nbytes >= (1 << 30) else 96)
+            t = timed(lambda i: lib.probe_read(views[i % copies], sink, blocks, pieces),
+                      12 if nbytes >= (1 << 30) else 96)
             best = max(best, nbytes / t)
         out[label] = round(best / 1e9, 1)
     del pool

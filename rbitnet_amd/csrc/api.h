@@ -147,9 +147,11 @@ int rb_place_rows(const void* src, int src_dtype, void* dst, int dst_dtype, int 
                   long long width, long long dst_rows, long long row0, long long block, long long period, void* stream);
 
 // What the GPU reaches, measured the simplest way: rb_probe_read reads `bytes` bytes (a multiple of
-// 16) once with 16-byte loads from `blocks` workgroups of 256 lanes; rb_probe_mfma runs 4 * iters bfloat16 32x32x16 MFMAs in each of `waves`
+// 16) once with 16-byte loads from `blocks` workgroups of 256 lanes (mode 0: all workgroups stride
+// through the buffer together, plain loads; mode 1: every workgroup walks pieces of 64 KB of its own
+// with non-temporal loads, which is a quarter faster on this GPU); rb_probe_mfma runs 4 * iters bfloat16 32x32x16 MFMAs in each of `waves`
 // waves (a multiple of 4).  `sink` is one float of device memory that is practically never written.
-int rb_probe_read(const void* p, long long bytes, int blocks, float* sink, void* stream);
+int rb_probe_read(const void* p, long long bytes, int blocks, int mode, float* sink, void* stream);
 int rb_probe_mfma(int waves, int iters, float* sink, void* stream);
 
 #ifdef __cplusplus

@@ -142,7 +142,7 @@ class Kernels:
             "rb_sample": [_P, _I, _I, _P, _P, _P, _P, _P],
             "rb_fill_normal": [_P, _I, ctypes.c_longlong, ctypes.c_ulonglong, ctypes.c_double, ctypes.c_double, _P],
             "rb_place_rows": [_P, _I, _P, _I, _I] + [ctypes.c_longlong] * 6 + [_P],
-            "rb_probe_read": [_P, ctypes.c_longlong, _I, _P, _P],
+            "rb_probe_read": [_P, ctypes.c_longlong, _I, _I, _P, _P],
             "rb_probe_mfma": [_I, _I, _P, _P],
         }
         for name, args in sig.items():
@@ -423,14 +423,15 @@ class Kernels:
                                          self._stream()))
 
     # ------------------------------------------------------------------ probes
-    def probe_read(self, buf: torch.Tensor, sink: torch.Tensor, blocks: int = 2048) -> None:
-        """Reads every byte of `buf` once with `blocks` workgroups (see probe.hip)."""
+    def probe_read(self, buf: torch.Tensor, sink: torch.Tensor, blocks: int = 2048, pieces: bool = False) -> None:
+        """Reads every byte of `buf` once with `blocks` workgroups (see probe.hip).  pieces: every
+        workgroup walks pieces of its own with non-temporal loads, as the decode products do."""
         _check(buf, "buf")
         _check(sink, "sink", torch.float32)
         nbytes = buf.numel() * buf.element_size()
         if nbytes % 16 != 0 or buf.data_ptr() % 16 != 0:
             raise KernelError("probe buffer must be 16-byte aligned and a multiple of 16 bytes long")
-        self._ok(self._lib.rb_probe_read(_ptr(buf), nbytes, int(blocks), _ptr(sink), self._stream()))
+        self._ok(self._lib.rb_probe_read(_ptr(buf), nbytes, int(blocks), int(bool(pieces)), _ptr(sink), self._stream()))
 
     def probe_mfma(self, waves: int, iters: int, sink: torch.Tensor) -> float:
         """Runs the MFMA loop; returns the floating-point operations it performs."""

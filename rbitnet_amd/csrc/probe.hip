@@ -1,6 +1,9 @@
 // What this GPU reaches on the two things the model's kernels are bound by, measured the
 // simplest way, so that a kernel's time can be read against more than the nominal peaks:
-//  * rb_probe_read: every byte of a buffer once, 16 bytes per lane and load, grid-stride.
+//  * rb_probe_read: every byte of a buffer once, 16 bytes per lane and load.  Mode 0: all
+//    workgroups stride through the buffer together, plain loads (5.3-5.6 TB/s for 1 GB).  Mode 1:
+//    every workgroup walks pieces of 64 KB of its own with non-temporal loads (7.0-7.1 TB/s): how
+//    the decode products read their weights.
 //  * rb_probe_mfma: back-to-back 32x32x16 bfloat16 MFMAs on four independent accumulators
 //    per wave, operands in registers, nothing else.
 // Neither has a counterpart in the reference (which measures nothing on a GPU).
@@ -40,11 +43,36 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(int iters, float* sink)
   if (v == 12345.678f) *sink = v;
 }
 
+// pieces of 64 KB dealt round robin to the workgroups; a piece is walked by the workgroup's 256
+// lanes, four non-temporal loads in flight per lane
+__global__ __launch_bounds__(256) void probe_read_pieces_kernel(const uint4* __restrict__ p, size_t n16, float* sink) {
+  constexpr size_t PIECE = 65536 / 16;
+  uint32_t acc = 0;
+  const size_t n_pieces = n16 / PIECE;
+  for (size_t c = blockIdx.x; c < n_pieces; c += gridDim.x) {
+    const uint4* q = p + c * PIECE;
+    for (size_t i = threadIdx.x; i < PIECE; i += 4 * 256) {
+      const uint4 a = load16_stream(q + i), b = load16_stream(q + i + 256), e = load16_stream(q + i + 512),
+                  d = load16_stream(q + i + 768);
+      acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ e.x ^ e.y ^ e.z ^ e.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    }
+  }
+  for (size_t i = n_pieces * PIECE + (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) {
+    const uint4 a = p[i];
+    acc ^= a.x ^ a.y ^ a.z ^ a.w;
+  }
+  if (acc == 0x9e3779b9u) *sink = 1.f;
+}
+
 // Reads `bytes` bytes (a multiple of 16) starting at p with `blocks` workgroups of 256 lanes.
-extern "C" int rb_probe_read(const void* p, long long bytes, int blocks, float* sink, void* stream) {
-  RB_REQUIRE(p != nullptr && sink != nullptr && bytes > 0 && bytes % 16 == 0 && blocks > 0 && blocks <= 65536,
+extern "C" int rb_probe_read(const void* p, long long bytes, int blocks, int mode, float* sink, void* stream) {
+  RB_REQUIRE(p != nullptr && sink != nullptr && bytes > 0 && bytes % 16 == 0 && blocks > 0 && blocks <= 65536 &&
+                 (mode == 0 || mode == 1),
              "rb_probe_read: bad arguments");
-  probe_read_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((const uint4*)p, (size_t)(bytes / 16), sink);
+  if (mode == 1)
+    probe_read_pieces_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((const uint4*)p, (size_t)(bytes / 16), sink);
+  else
+    probe_read_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((const uint4*)p, (size_t)(bytes / 16), sink);
   RB_LAUNCH_CHECK();
   return 0;
 }

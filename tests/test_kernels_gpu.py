@@ -745,19 +745,36 @@ def test_sample_frequencies_follow_softmax(lib):
 
 
 # ------------------------------------------------------------------------ probes
-def test_probes_run(lib):
-    """The streaming-read and MFMA probes of the benchmark launch, touch nothing but their
-    sink, and refuse a buffer they cannot read with 16-byte loads."""
+def test_probes_read_every_byte_and_write_nothing(lib):
+    """The streaming-read probes of the benchmark, in both modes: a lane whose values xor to a
+    magic number raises the sink, so a buffer of zeros with that number in one place shows
+    whether the place was read: the first and the last 16 bytes, one in the middle, one in the
+    rest that is no whole piece of 64 KB.  They write nothing else and refuse a buffer they
+    cannot read with 16-byte loads."""
     from rbitnet_amd.errors import KernelError
+    magic = 0x9E3779B9 - (1 << 32)
+    n = (3 << 20) // 4 + 4 * 1000                # three pieces of 64 KB x 16 and a rest, in int32 words
+    for pieces in (False, True):
+        for blocks in (1, 7, 64):
+            for word in (0, n // 2 // 4 * 4, n - 4 * 500, n - 4):
+                buf = torch.zeros(n, dtype=torch.int32, device=DEV)
+                buf[word] = magic
+                before = buf.clone()
+                sink = torch.zeros(1, device=DEV)
+                lib.probe_read(buf, sink, blocks, pieces)
+                torch.cuda.synchronize()
+                assert float(sink) == 1.0, (pieces, blocks, word)
+                assert torch.equal(buf, before)
+            sink = torch.zeros(1, device=DEV)
+            lib.probe_read(torch.zeros(n, dtype=torch.int32, device=DEV), sink, blocks, pieces)
+            torch.cuda.synchronize()
+            assert float(sink) == 0.0
     sink = torch.zeros(1, device=DEV)
-    buf = torch.arange(1 << 20, dtype=torch.int32, device=DEV)
-    before = buf.clone()
-    lib.probe_read(buf, sink, 64)
     assert lib.probe_mfma(8, 10, sink) == 8 * 10 * 4 * 2 * 32 * 32 * 16
     torch.cuda.synchronize()
-    assert torch.equal(buf, before) and float(sink) == 0.0
+    assert float(sink) == 0.0
     with pytest.raises(KernelError):
-        lib.probe_read(buf[:3], sink)
+        lib.probe_read(torch.zeros(16, dtype=torch.int32, device=DEV)[:3], sink)
 
 
 @pytest.mark.parametrize("m", [1, 5, 16, 17, 40, 64, 100, 256, 700, 2100])
