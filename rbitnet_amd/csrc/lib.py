@@ -15,6 +15,7 @@ import torch
 from ..errors import KernelError
 from . import build as _build
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _F32, _BF16 = 0, 1
 _P = ctypes.c_void_p
 _I = ctypes.c_int
@@ -160,11 +161,17 @@ class Kernels:
             for name in TIMED_OPS:
                 setattr(self, name, self.times.wrap(name, getattr(self, name)))
             atexit.register(lambda: print(self.times.report(), file=sys.stderr, flush=True))
+        self.device_index = int(torch.cuda.current_device())
         self.n_compute_units = int(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count)
 
     # ------------------------------------------------------------------ helpers
-    @staticmethod
-    def _stream() -> int:
+    def _stream(self) -> int:
+        """torch's current HIP stream of this GPU, as a raw handle.  Asked for at every launch (a
+        step that is being captured runs on another stream than the one before it), through torch's
+        own fast path where it has one: `torch.cuda.current_stream()` builds a Python object at
+        8 us a call, a third of what a launch costs on the host."""
+        if _RAW_STREAM is not None:
+            return _RAW_STREAM(self.device_index)
         return torch.cuda.current_stream().cuda_stream
 
     def _ok(self, rc: int) -> None:
