@@ -691,6 +691,10 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
   // for the caches to matter (batch 64: 1.9 % of the step, batch 8: 0.8 %; with a single sequence
   // the plain loads are 1.2 % faster).
   const bool v_once = gridDim.y * gridDim.z >= 32;
+  // The keys likewise where the launch is large (512 workgroups and more: batch 64 at 8,192 keys 4.7 %
+  // of the step, at 530 keys 1.9 %, batch 8 at 32,768 keys 1-5 %); in small launches, which wait for
+  // their first page rather than for bandwidth, they lose (batch 8 at 530 keys: 0.9 %).
+  const bool k_once = gridDim.x * gridDim.y * gridDim.z >= 512;
   auto ask_values = [&](int page) {        // into this wave's area of LDS
     const bf16_t* rows = v_pages + ((size_t)page * n_kv + kvh) * RB_PAGE * D;
 #pragma unroll
@@ -706,7 +710,10 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int st = 0; st < KS; ++st) kf_next[t][st].u = load16(rows + (size_t)(16 * t + c16) * D + 32 * st + 8 * grp);
+      for (int st = 0; st < KS; ++st) {
+        const bf16_t* src = rows + (size_t)(16 * t + c16) * D + 32 * st + 8 * grp;
+        kf_next[t][st].u = k_once ? load16_stream(src) : load16(src);
+      }
   };
 
   // ---- q of the group (rotated here when FUSED) as bfloat16 rows in LDS, zero rows beyond it

@@ -381,7 +381,8 @@ def decode_kernel(lib, request):
 
 
 _DECODE_CASES = [(4, 1, 128, 0, 3), (8, 8, 64, 0, 1), (8, 4, 128, 0, 8), (8, 1, 64, 90, 2), (2, 2, 128, 65, 5),
-                 (6, 2, 128, 0, 3), (16, 1, 64, 0, 2), (10, 2, 128, 70, 2), (7, 1, 64, 0, 4), (12, 1, 128, 130, 1)]
+                 (6, 2, 128, 0, 3), (16, 1, 64, 0, 2), (10, 2, 128, 70, 2), (7, 1, 64, 0, 4), (12, 1, 128, 130, 1),
+                 (8, 8, 128, 0, 16)]          # the last one: 768 workgroups, where keys are read past the caches
 
 
 @pytest.mark.parametrize("decode_kernel", ["auto", "matrix"], indirect=True)
