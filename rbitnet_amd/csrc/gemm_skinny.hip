@@ -339,9 +339,8 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(const bf16_t* __restri
   }
 }
 
-static int g_tune_u = 0, g_tune_r = 0, g_tune_waves = 0;
-extern "C" void rb_tune(int u, int r, int waves) {       // experiments only; 0 = the built-in choice
-  g_tune_u = u;
+static int g_tune_r = 0, g_tune_waves = 0;
+extern "C" void rb_tune(int r, int waves) {       // experiments only; 0 = the built-in choice
   g_tune_r = r;
   g_tune_waves = waves;
 }
@@ -603,11 +602,7 @@ __global__ __launch_bounds__(512) void gemm_resident_kernel(const bf16_t* __rest
 }
 
 static int g_res_tiles = 0;
-extern "C" void rb_tune_resident(int waves, int parts, int tiles) {      // experiments only; 0 = built-in
-  (void)waves;
-  (void)parts;
-  g_res_tiles = tiles;
-}
+extern "C" void rb_tune_resident(int tiles) { g_res_tiles = tiles; }      // experiments only; 0 = built-in
 
 template <int MB, int XQ, int EPI, typename TO, bool SCALED>
 static int launch_resident(const GemmTokens& x, const bf16_t* w, void* c, const GemmAfter& after, int m, int n, int k,

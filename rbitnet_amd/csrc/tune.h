@@ -8,8 +8,8 @@
 extern "C" {
 #endif
 
-void rb_tune(int stages, int rows_per_wave, int waves);         // skinny product
-void rb_tune_resident(int waves, int parts, int tiles);         // skinny product with resident tokens
+void rb_tune(int rows_per_wave, int waves);                     // skinny product
+void rb_tune_resident(int tiles);                               // skinny product with resident tokens: row tiles per workgroup
 void rb_tune_use_resident(int on);                              // 0: never the resident variant, 2: also below 8192 rows
 void rb_tune_use_stream(int on);                                // 0: the skinny product up to 64 tokens
 void rb_tune_tiles(int cfg, int parts);                         // tiled product: tile configuration and K slices
