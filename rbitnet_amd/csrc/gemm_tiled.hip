@@ -331,7 +331,9 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   // workgroup's walk along K is long: the short walks of a product cut into many K slices are
   // bound by their first loads, which come sooner through the caches (64 tokens: 28,672 gated rows
   // 51 -> 43 us with such loads, but 4,096 rows in 8 slices of 8 tiles 15 -> 16.6 us).
-  const bool w_once = WF && m_tiles == 1 && k_tiles >= 24;
+  // (only in the kernels with tiles of at most 128 tokens: in the others the choice would stand as
+  // branches between the MFMAs of the main loop)
+  const bool w_once = WF && BM <= 128 && m_tiles == 1 && k_tiles >= 24;
   auto issue = [&](int kt) {
     const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
     const uint32_t kbytes = (uint32_t)(kt0 + kt) * (BK * 2);
