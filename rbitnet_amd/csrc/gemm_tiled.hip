@@ -659,6 +659,11 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   // 128 x 128 tiles; at K = 4096, 768 tokens by 4,096 rows 46 against 59, 512 by 6,144 48 against 56.
   // 160 workgroups of 2 slices still win (640 tokens by 4,096 rows: 43 against 58), 144 do not.
   const long long t256x128 = (long long)((m + 127) / 128) * ((n + 255) / 256);
+  // A deep product (K >= 8192) whose 256 x 256 tiles are half a round goes in 2 slices of those
+  // rather than in one round of the 256 x 128 tiles (4,096 rows at K = 14336: 2,048 tokens 197 us
+  // against 220, 1,536 tokens 172 against 195; the second slab costs the norm that adds it about 10).
+  if (m > 64 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 64 && t256 * 2 >= 192 && t256 * 2 <= 256)
+    return {4, 2};
   if (m > 64 && t256x128 >= 192 && t256x128 <= 256) return {8, 1};
   if (m > 64 && epilogue == 0) {
     for (int p = 2; p <= 4; p *= 2)
