@@ -638,13 +638,14 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   const long long t64 = (long long)((m + 63) / 64) * ((n + 127) / 128);
   if (m > 64 && t256 >= 160) {
     // rounds of 256 workgroups times the time of a tile: a 192-row tile does 0.75 of the work
-    // of a 256-row one in 0.81 of the time, a 320-row tile 1.25 of it in 1.26 (28,672 gated rows
-    // by 2,048 tokens: 896 tiles of 256 rows, 3.5 rounds, 475 us; 720 of 320 rows, under 3
-    // rounds, 459 us)
+    // of a 256-row one in 0.81 of the time, a 320-row tile 1.25 of it in 1.22 to 1.26 (28,672 gated
+    // rows by 2,048 tokens: 896 tiles of 256 rows, 3.5 rounds, 475 us; 720 of 320 rows, under 3
+    // rounds, 459 us).  Checked against the fastest of the three for 28,672 gated rows at 384 to
+    // 4,096 tokens in steps of 128, and for 6,144 and 4,096 rows: within 2 % everywhere.
     const long long t192 = (long long)((m + 255) / 256) * ((n + 191) / 192);
     const long long t320 = (long long)((m + 255) / 256) * ((n + 319) / 320);
     const long long cost256 = (t256 + 255) / 256 * 1000, cost192 = (t192 + 255) / 256 * 815,
-                    cost320 = (t320 + 255) / 256 * 1260;
+                    cost320 = (t320 + 255) / 256 * 1220;
     if (cost320 < cost256 && cost320 < cost192) return {9, 1};
     return {cost192 < cost256 ? 6 : 4, 1};
   }
@@ -653,7 +654,8 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   // unit, 2,048 tokens by 4,096 rows 237 us against 258 at K = 14336 and 82.6 against 83.6 at
   // K = 4096; 1,024 tokens by 6,144 rows 76 against 82; 256 tokens by 28,672 gated rows 80 against
   // 89.  With fewer or more tiles than that they lose (1,024 tokens by 4,096 rows: 204 against 159).
-  // Where they are half or a quarter of a round, K is cut into 2 or 4 slices of at least 32 tiles,
+  // Where they are half, a quarter or an eighth of a round, K is cut into 2, 4 or 8 slices of at least 32
+  // (8 slices: 24) tiles (256 tokens by 4,096 rows at K = 14336: 41 us in 8 slices against 59),
   // which fills the round again: 512 tokens by 4,096 rows at K = 14336 75 us in 4 slices against 107
   // in the 64-token tiles (320 tokens: 64 against 106), 1,024 tokens 127 in 2 slices against 146 in
   // 128 x 128 tiles; at K = 4096, 768 tokens by 4,096 rows 46 against 59, 512 by 6,144 48 against 56.
@@ -664,10 +666,15 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   // against 220, 1,536 tokens 172 against 195; the second slab costs the norm that adds it about 10).
   if (m > 64 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 64 && t256 * 2 >= 192 && t256 * 2 <= 256)
     return {4, 2};
+  // and where they are a quarter of a round, in 4 slices (768 tokens: 94 us against 106 in 2 slices of the
+  // 256 x 128 tiles; 1,024 tokens: 109 against 118)
+  if (m > 64 && epilogue == 0 && (k / 64) % 4 == 0 && k / 64 / 4 >= 48 && t256 * 4 >= 192 && t256 * 4 <= 256)
+    return {4, 4};
   if (m > 64 && t256x128 >= 192 && t256x128 <= 256) return {8, 1};
   if (m > 64 && epilogue == 0) {
-    for (int p = 2; p <= 4; p *= 2)
-      if (t256x128 * p >= 160 && t256x128 * p <= 256 && (k / 64) % p == 0 && k / 64 / p >= 32) return {8, p};
+    for (int p = 2; p <= 8; p *= 2)
+      if (t256x128 * p >= 160 && t256x128 * p <= 256 && (k / 64) % p == 0 && k / 64 / p >= (p == 8 ? 24 : 32))
+        return {8, p};
   }
   // Between one and two thousand tokens the large tiles are too few for a round by themselves: a deep
   // product (K >= 8192) is cut into 2 slices of them (1,152 tokens by 4,096 rows at K = 14336: 164 us in
