@@ -183,19 +183,38 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     if (next) load_tile(kt + 1);
     if (wave_on && kt >= wave_first && kt <= wave_last) {
 
-    // ---- S^T = K Q^T: rows keys, columns queries
+    // ---- S^T = K Q^T: rows keys, columns queries.  The fragments of K come from LDS a few MFMAs
+    // ahead of their use, one read behind every MFMA: left to itself the compiler asked for two
+    // and waited for them before every second MFMA, and a wave alone on its SIMD took 2.1 us a
+    // tile where its 32 MFMAs take 0.55.
+    constexpr int AHEAD = 4;                     // fragments on their way
+    constexpr int SD = D / 16;                   // depth steps of the scores
     f32x16_t sacc[2];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
+    for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
       for (int e = 0; e < 16; ++e) sacc[rt][e] = 0.f;
+    Frag8 ring[AHEAD];
+    auto k_read = [&](int f) {                   // fragment f: row tile f / SD, depth step f % SD
+      ring[f % AHEAD].u = *reinterpret_cast<const uint4*>(ks + ((f / SD) * 32 + l32) * KLD + (f % SD) * 16 + g * 8);
+    };
 #pragma unroll
-      for (int s = 0; s < D / 16; ++s) {
-        Frag8 a;
-        a.u = *reinterpret_cast<const uint4*>(ks + (rt * 32 + l32) * KLD + s * 16 + g * 8);
-        sacc[rt] = mfma32(a, qf[s], sacc[rt]);
-      }
+    for (int f = 0; f < AHEAD; ++f) k_read(f);
+#pragma unroll
+    for (int f = 0; f < 2 * SD; ++f) {
+      sacc[f / SD] = mfma32(ring[f % AHEAD], qf[f % SD], sacc[f / SD]);
+      if (f + AHEAD < 2 * SD) k_read(f + AHEAD);
+      __builtin_amdgcn_sched_barrier(0);
     }
+    // the first fragments of V^T are asked for now and arrive during the softmax arithmetic:
+    // fragment f belongs to step f / VD (row tile and half, see below) and d tile f % VD
+    constexpr int VD = D / 32;
+    auto v_read = [&](int f) {
+      const int q = f / VD, i = f % VD;
+      ring[f % AHEAD].u = *reinterpret_cast<const uint4*>(vt + (i * 32 + l32) * VLD + (q / 2) * 32 + (2 * (q % 2) + g) * 8);
+    };
+#pragma unroll
+    for (int f = 0; f < AHEAD; ++f) v_read(f);
     // ---- mask (only tiles that touch the diagonal or the window's edge), running maximum.
     // Scores stay unscaled: the scale is positive, so the maximum can be taken first and the
     // scale folded into the exponent's argument.
@@ -243,22 +262,22 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     // ---- O^T += V^T P^T.  Step (rt, mm) takes the 16 keys whose probabilities sit in
     // registers 8 mm .. 8 mm + 7 of row tile rt: for lane group g these are keys
     // 32 rt + 16 mm + 8 h + 4 g + e (h = 0, 1; e = 0..3), and V^T was stored in that order.
+    Frag8 pb[4];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
+    for (int q = 0; q < 4; ++q) {
+      const int rt = q / 2, mm = q % 2;
+      pb[q].u.x = pack_bf16x2(sacc[rt][8 * mm + 0], sacc[rt][8 * mm + 1]);
+      pb[q].u.y = pack_bf16x2(sacc[rt][8 * mm + 2], sacc[rt][8 * mm + 3]);
+      pb[q].u.z = pack_bf16x2(sacc[rt][8 * mm + 4], sacc[rt][8 * mm + 5]);
+      pb[q].u.w = pack_bf16x2(sacc[rt][8 * mm + 6], sacc[rt][8 * mm + 7]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int mm = 0; mm < 2; ++mm) {
-        Frag8 pb;
-        pb.u.x = pack_bf16x2(sacc[rt][8 * mm + 0], sacc[rt][8 * mm + 1]);
-        pb.u.y = pack_bf16x2(sacc[rt][8 * mm + 2], sacc[rt][8 * mm + 3]);
-        pb.u.z = pack_bf16x2(sacc[rt][8 * mm + 4], sacc[rt][8 * mm + 5]);
-        pb.u.w = pack_bf16x2(sacc[rt][8 * mm + 6], sacc[rt][8 * mm + 7]);
-#pragma unroll
-        for (int i = 0; i < D / 32; ++i) {
-          Frag8 a;
-          a.u = *reinterpret_cast<const uint4*>(vt + (i * 32 + l32) * VLD + rt * 32 + (2 * mm + g) * 8);
-          oacc[i] = mfma32(a, pb, oacc[i]);
-        }
-      }
+    for (int f = 0; f < 4 * VD; ++f) {
+      oacc[f % VD] = mfma32(ring[f % AHEAD], pb[f / VD], oacc[f % VD]);
+      if (f + AHEAD < 4 * VD) v_read(f + AHEAD);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     }
     if (next) store_tile(buf ^ 1);
     __syncthreads();
