@@ -390,13 +390,26 @@ static int dispatch_skinny(const GemmTokens& x, const bf16_t* w, void* c, const 
   const int mb = (m + 15) / 16;
   RB_REQUIRE(!FOLDS || mb == 1, "rb_gemm_bf16: a product that folds its neighbours in takes at most 16 tokens, not %d",
              m);
-  // Row tiles of W per wave (16 R rows per workgroup).  Measured with 8 tokens, W fragment-major, N from
-  // 1024 to 16384: up to K = 4096 (workgroups of 4 waves, several of which share a compute unit) one tile
-  // per wave is the fastest at every N (N = 6144: 11.1 us against 13.5 with two); from K = 8192 on
-  // (8 waves) one tile as long as that gives every compute unit one workgroup at most, two beyond
-  // (K = 8192, N = 6144: 24.3 us with one, 21.1 with two).  Four never won below the row counts that the
-  // token-resident kernel takes.
-  int r = (k < 8192 || (n + 15) / 16 <= 256) ? 1 : 2;
+  // Row tiles of W per wave (16 R rows per workgroup).  Up to K = 4096 (workgroups of 4 waves, several
+  // of which share a compute unit) one tile per wave is the fastest at every N from 1024 to 16384
+  // (measured with 8 tokens, W fragment-major; N = 6144: 11.1 us against 13.5 with two).  From
+  // K = 8192 on (8 waves) more tiles reuse the token operand better and fewer deal the rows to the 256
+  // compute units more evenly: the time goes with the rows that the busiest compute unit gets, at
+  // a price per row that falls with R (about 15 % / R).  57344 rows at K = 8192: R = 4 gives 896
+  // workgroups, 4 on some compute units and 3 on others, 194 us; R = 2 gives every one 7: 175 us.
+  // 10240 rows at K = 8192 with one token: R = 1 35 us, R = 2 42.
+  int r = 1;
+  if (k >= 8192) {
+    double best = 0.0;
+    for (int cand = (EPI == 1 ? 2 : 1); cand <= 4; cand *= 2) {
+      const long long wgs = (n + 16 * cand - 1) / (16 * cand);
+      const double cost = (double)((wgs + 255) / 256 * 16 * cand) * (1.0 + 0.15 / cand);
+      if (best == 0.0 || cost <= best) {
+        best = cost;
+        r = cand;
+      }
+    }
+  }
   if (g_tune_r) r = g_tune_r;
   if (EPI == 1 && r < 2) r = 2;
 #define RB_SK(MBV, RV) return launch_skinny_u<MBV, RV, EPI, TO, SCALED>(x, w, c, after, m, n, k, s)
