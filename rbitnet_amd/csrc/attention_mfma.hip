@@ -661,7 +661,7 @@ __device__ __forceinline__ int v_swizzle(int key) {
   return D == 128 ? ((key & 7) << 1) : (((key >> 1) & 3) << 1);
 }
 
-template <int D, int NW, bool FUSED>
+template <int D, int NW, bool FUSED, int ONCE>
 __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
     const float* __restrict__ qkv, const bf16_t* __restrict__ q_in, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int style, bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out,
@@ -706,21 +706,17 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
   int id_after = pg_first + pg_step <= last_page ? pages[pg_first + pg_step] : 0;  // the one after it
   uint16_t* vpage = vpages + wave * RB_PAGE * D;
   const uint32_t vpage_lds = (uint32_t)(uintptr_t)vpage;
-  // A page of V is whole rows, read once in a step: past the caches when the batch is large enough
-  // for the caches to matter (batch 64: 1.9 % of the step, batch 8: 0.8 %; with a single sequence
-  // the plain loads are 1.2 % faster).
-  const bool v_once = gridDim.y * gridDim.z >= 32;
-  // The keys likewise where the launch is large (512 workgroups and more: batch 64 at 8,192 keys 4.7 %
-  // of the step, at 530 keys 1.9 %, batch 8 at 32,768 keys 1-5 %); in small launches, which wait for
-  // their first page rather than for bandwidth, they lose (batch 8 at 530 keys: 0.9 %).
-  const bool k_once = gridDim.x * gridDim.y * gridDim.z >= 512;
+  // ONCE >= 1: the pages of V, whole rows that are read once in a step, go past the caches; ONCE = 2: the
+  // keys as well (the launcher says when).  Compiled in: as a run-time choice it stood as a branch at
+  // every load of a page.
+  constexpr bool v_once = ONCE >= 1, k_once = ONCE >= 2;
   auto ask_values = [&](int page) {        // into this wave's area of LDS
     const bf16_t* rows = v_pages + ((size_t)page * n_kv + kvh) * RB_PAGE * D;
 #pragma unroll
     for (int i = 0; i < VI; ++i) {
       const int key = i * RPI + lane / CPR;
       const int chunk = (lane % CPR) ^ v_swizzle<D>(key);
-      if (v_once) load_to_lds16_stream(rows, (uint32_t)(key * D + chunk * 8) * 2u, vpage_lds + i * 1024u);
+      if constexpr (v_once) load_to_lds16_stream(rows, (uint32_t)(key * D + chunk * 8) * 2u, vpage_lds + i * 1024u);
       else load_to_lds16(rows, (uint32_t)(key * D + chunk * 8) * 2u, vpage_lds + i * 1024u);
     }
   };
@@ -731,7 +727,8 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
 #pragma unroll
       for (int st = 0; st < KS; ++st) {
         const bf16_t* src = rows + (size_t)(16 * t + c16) * D + 32 * st + 8 * grp;
-        kf_next[t][st].u = k_once ? load16_stream(src) : load16(src);
+        if constexpr (k_once) kf_next[t][st].u = load16_stream(src);
+        else kf_next[t][st].u = load16(src);
       }
   };
 
@@ -1003,10 +1000,10 @@ static void launch_decode(const DecodeArgs& a, hipStream_t s) {
   if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits);
 }
 
-template <int D, int NW, bool FUSED>
+template <int D, int NW, bool FUSED, int ONCE>
 static int launch_decode_mfma_nw(const DecodeArgs& a, hipStream_t s) {
   const size_t lds = (size_t)NW * RB_PAGE * D * 2 + 16 * D * 2 + 2 * D * 2 + (size_t)NW * (16 + 64) * sizeof(float);
-  auto kern = attn_decode_mfma_kernel<D, NW, FUSED>;
+  auto kern = attn_decode_mfma_kernel<D, NW, FUSED, ONCE>;
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1032,7 +1029,20 @@ template <int D, bool FUSED>
 static int launch_decode_mfma(const DecodeArgs& a, hipStream_t s) {
   const long long wgs = (long long)a.n_splits * a.n_kv * a.n_seqs;
   const int nw = g_decode_waves ? g_decode_waves : (wgs <= 256 && a.n_splits == 1 ? 8 : 4);
-  return nw == 8 ? launch_decode_mfma_nw<D, 8, FUSED>(a, s) : launch_decode_mfma_nw<D, 4, FUSED>(a, s);
+  // Pages past the caches.  V when the batch is large enough for the caches to matter (32 sequences x
+  // kv heads and more: batch 64 1.9 % of the step, batch 8 0.8 %; with a single sequence the plain loads
+  // are 1.2 % faster).  The keys as well where the launch is large (512 workgroups and more: batch 64
+  // at 8,192 keys 4.7 % of the step, at 530 keys 1.9 %); in small launches, which wait for their first
+  // page rather than for bandwidth, they lose (batch 8 at 530 keys: 0.9 %).
+  const int once = (long long)a.n_kv * a.n_seqs < 32 ? 0 : (wgs >= 512 ? 2 : 1);
+  if (nw == 8) {
+    if (once == 0) return launch_decode_mfma_nw<D, 8, FUSED, 0>(a, s);
+    if (once == 1) return launch_decode_mfma_nw<D, 8, FUSED, 1>(a, s);
+    return launch_decode_mfma_nw<D, 8, FUSED, 2>(a, s);
+  }
+  if (once == 0) return launch_decode_mfma_nw<D, 4, FUSED, 0>(a, s);
+  if (once == 1) return launch_decode_mfma_nw<D, 4, FUSED, 1>(a, s);
+  return launch_decode_mfma_nw<D, 4, FUSED, 2>(a, s);
 }
 
 // Which decode kernel: 0 = by group size (matrix cores from 2 query heads per kv head on: the

@@ -6,6 +6,8 @@
 // silu(gate) * up (llama/model.rs:297-302 of the reference) instead of the two products.
 //
 // Reference loop: y[o] = sum_i W[i + o * n_in] * x[i]  (llama/model.rs:67-91).
+#include <type_traits>
+
 #include "api.h"
 #include "tune.h"
 #include "gemm_internal.h"
@@ -331,15 +333,15 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   // workgroup's walk along K is long: the short walks of a product cut into many K slices are
   // bound by their first loads, which come sooner through the caches (64 tokens: 28,672 gated rows
   // 51 -> 43 us with such loads, but 4,096 rows in 8 slices of 8 tiles 15 -> 16.6 us).
-  // (only in the kernels with tiles of at most 128 tokens: in the others the choice would stand as
-  // branches between the MFMAs of the main loop)
-  const bool w_once = WF && BM <= 128 && m_tiles == 1 && k_tiles >= 24;
-  auto issue = [&](int kt) {
+  // The main loop is compiled for either kind of load (as a run-time choice it stood as eight branches
+  // between the MFMAs of a K tile and cost 1.6 % of a long prefill).
+  const bool w_once = WF && m_tiles == 1 && k_tiles >= 24;
+  auto issue = [&](auto once, int kt) {
     const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
     const uint32_t kbytes = (uint32_t)(kt0 + kt) * (BK * 2);
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i) {
-      if (w_once)
+      if constexpr (decltype(once)::value)
         load_to_lds16_stream(wtile, woff[i] + (uint32_t)(kt0 + kt) * W_KSTEP,
                              stage + (uint32_t)(wave + NWAVES * i) * 1024u);
       else
@@ -386,19 +388,12 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   // of tile kt, whose fragments are in registers by then: its MFMAs run while the first
   // fragments of tile kt + 1 come from LDS and while the other waves arrive, and the stage of
   // tile kt is free for tile kt + S from there on.
-#pragma unroll
-  for (int s = 0; s < S; ++s)
-    if (s < k_tiles) issue(s);
-  if (S - 1 < k_tiles) wait_vm<LOADS * (S - 1)>();
-  else wait_vm<0>();
-  __syncthreads();
-  load_frags(0, 0, 0);
   // One load of tile kt (number l of the LOADS a wave has), one fragment of a depth step.
-  auto issue_one = [&](int kt, int l) {
+  auto issue_one = [&](auto once, int kt, int l) {
     const uint32_t stage = lds_base + (uint32_t)(kt % S) * (STAGE * 2);
     const uint32_t kbytes = (uint32_t)(kt0 + kt) * (BK * 2);
     if (l < W_LOADS) {
-      if (w_once)
+      if constexpr (decltype(once)::value)
         load_to_lds16_stream(wtile, woff[l] + (uint32_t)(kt0 + kt) * W_KSTEP,
                              stage + (uint32_t)(wave + NWAVES * l) * 1024u);
       else
@@ -440,13 +435,13 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
   // loads of tile kt + S and the first fragments of tile kt + 1, so that the matrix core never
   // waits for a run of other instructions (both waves of a SIMD leave the barrier together, and
   // neither covers the other's).
-  auto last_step = [&](int kt, bool fetch) {
+  auto last_step = [&](auto once, int kt, bool fetch) {
 #pragma unroll
     for (int q = 0; q < NM; ++q) {
       acc[q / TM][q % TM] = mfma32(b[LASTBUF][q % TM], a[LASTBUF][q / TM], acc[q / TM][q % TM]);
       if (fetch) {
 #pragma unroll
-        for (int l = q; l < LOADS; l += NM) issue_one(kt + S, l);
+        for (int l = q; l < LOADS; l += NM) issue_one(once, kt + S, l);
       }
 #pragma unroll
       for (int f = q; f < TN + TM; f += NM) frag_one(0, kt + 1, 0, f);
@@ -462,19 +457,30 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
     __syncthreads();                  // everyone's part of tile kt + 1 is in LDS, and nobody reads tile kt's stage any more
     __builtin_amdgcn_sched_barrier(0);
   };
-  int kt = 0;
-  for (; kt + S < k_tiles; ++kt) {
-    steps_but_last(kt);
-    hand_over(kt);
-    last_step(kt, true);
-  }
-  for (; kt + 1 < k_tiles; ++kt) {
-    steps_but_last(kt);
-    hand_over(kt);
-    last_step(kt, false);
-  }
-  steps_but_last(k_tiles - 1);
-  mfmas(LASTBUF);
+  auto run = [&](auto once) {
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+      if (s < k_tiles) issue(once, s);
+    if (S - 1 < k_tiles) wait_vm<LOADS * (S - 1)>();
+    else wait_vm<0>();
+    __syncthreads();
+    load_frags(0, 0, 0);
+    int kt = 0;
+    for (; kt + S < k_tiles; ++kt) {
+      steps_but_last(kt);
+      hand_over(kt);
+      last_step(once, kt, true);
+    }
+    for (; kt + 1 < k_tiles; ++kt) {
+      steps_but_last(kt);
+      hand_over(kt);
+      last_step(once, kt, false);
+    }
+    steps_but_last(k_tiles - 1);
+    mfmas(LASTBUF);
+  };
+  if (w_once) run(std::true_type{});
+  else run(std::false_type{});
 
   // ---- lane holds, per (i, j): W row n0 + wn0 + 32 i + l32, tokens base + 8 (e / 4) + 4 g + e % 4
   if constexpr (EPI == 1 && sizeof(TO) == 2) {
