@@ -660,8 +660,10 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   // unit, 2,048 tokens by 4,096 rows 237 us against 258 at K = 14336 and 82.6 against 83.6 at
   // K = 4096; 1,024 tokens by 6,144 rows 76 against 82; 256 tokens by 28,672 gated rows 80 against
   // 89.  With fewer or more tiles than that they lose (1,024 tokens by 4,096 rows: 204 against 159).
-  // Where they are half, a quarter or an eighth of a round, K is cut into 2, 4 or 8 slices of at least 32
-  // (8 slices: 24) tiles (256 tokens by 4,096 rows at K = 14336: 41 us in 8 slices against 59),
+  // Where they are half, a quarter or an eighth of a round, K is cut into 2, 4 or 8 slices of at least 32,
+  // 16 and 24 tiles (256 tokens by 4,096 rows at K = 14336: 41 us in 8 slices against 59; at K = 4096 in
+  // 4 slices, 512 tokens by 4,096 rows 24 us against 30, 256 by 6,144 24 against 30; 128 by 12,288 28 against 33,
+  // but there the four slabs cost the kernel that adds them more than that),
   // which fills the round again: 512 tokens by 4,096 rows at K = 14336 75 us in 4 slices against 107
   // in the 64-token tiles (320 tokens: 64 against 106), 1,024 tokens 127 in 2 slices against 146 in
   // 128 x 128 tiles; at K = 4096, 768 tokens by 4,096 rows 46 against 59, 512 by 6,144 48 against 56.
@@ -679,7 +681,7 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   if (m > 64 && t256x128 >= 192 && t256x128 <= 256) return {8, 1};
   if (m > 64 && epilogue == 0) {
     for (int p = 2; p <= 8; p *= 2)
-      if (t256x128 * p >= 160 && t256x128 * p <= 256 && (k / 64) % p == 0 && k / 64 / p >= (p == 8 ? 24 : 32))
+      if (t256x128 * p >= 160 && t256x128 * p <= 256 && (k / 64) % p == 0 && k / 64 / p >= (p == 2 ? 32 : (p == 4 ? (n <= 8192 ? 16 : 32) : 24)))
         return {8, p};
   }
   // Between one and two thousand tokens the large tiles are too few for a round by themselves: a deep
