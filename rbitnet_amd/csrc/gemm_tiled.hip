@@ -703,15 +703,20 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
     if (m <= 24) return {10, 1};
     if (k % 128 == 0) return {13, 1};
   }
-  // A short product (K <= 4096, up to 8,192 rows) of at most 64 tokens: tiles of 64 rows, four stages
-  // deep, two to a compute unit, in as many K slices as make up to 256 workgroups (64 tokens by 4,096 rows
-  // at K = 4096: 9.8 us in 4 slices against 11.1-12.9 in 8 slices of 128-row tiles; 6,144 rows: 13.4 in 2
-  // against 14.2 in 4), and the kernel that adds the slabs has half as many to add.
-  if (m <= 64 && epilogue == 0 && k <= 4096 && n <= 8192) {
-    const long long t64r = (n + 63) / 64;
-    int p = 1;
-    while (p < 8 && t64r * (2 * p) <= 256 && (k / 64) % (2 * p) == 0) p *= 2;
-    if (t64r * p >= 128) return {10, p};
+  // At most 64 tokens, no gate: tiles of 128 rows in K slices, or tiles of 64 rows (four stages deep, two
+  // to a compute unit) in half as many slices.  The small tiles where they make more workgroups, up to
+  // one per compute unit (4,096 rows at K = 11008, whose 172 K tiles go in 4 slices and not in 8: 19.5 us
+  // in 256 workgroups against 26.6 in 128), and at equal numbers where K is short (K = 4096: 4,096 rows
+  // 9.8 us in 4 slices against 11.1-12.9 in 8, 6,144 rows 13.4 against 14.2; K = 8192: 8,192 rows 24.9
+  // against 26.0): the kernel that adds the slabs then has half as many to add.  With a long K the
+  // large tiles win at equal numbers (4,096 rows at K = 14336: 22.2 us against 23.3), and so they do
+  // against small tiles in one slice (10,240 rows at K = 8192: 35.3 against 40.2).
+  if (m <= 64 && epilogue == 0) {
+    const int pa = k_slices(t64, k, 256, k / (8 * m));
+    const int pb = k_slices((n + 63) / 64, k, 256, 8);
+    const long long wa = t64 * pa, wb = (long long)((n + 63) / 64) * pb;
+    if (wb <= 256 && (wb > wa || (wb == wa && pb >= 2 && k <= 8192))) return {10, pb};
+    return {7, pa};
   }
   return {7, epilogue ? 1 : k_slices(t64, k, 256, k / (8 * m))};
 }
