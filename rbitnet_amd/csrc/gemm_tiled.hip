@@ -642,6 +642,16 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   }
   const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
   const long long t64 = (long long)((m + 63) / 64) * ((n + 127) / 128);
+  // Rows that divide into 320-row tiles exactly, in a deep product: those tiles in 2 or 4 K slices where that
+  // makes one round (10,240 rows at K = 8192: 512 tokens 77 us in 4 slices against 100 in 2 slices of
+  // 256 x 128 tiles, 1,024 tokens 135 in 2 slices against 180 in one round of 216 tiles of 192 rows).
+  // Only with tiles of tokens that are nearly full and a round that is nearly full (768 tokens, 192
+  // workgroups: slower than one round of the 256 x 128 tiles).
+  if (m > 64 && epilogue == 0 && n % 320 == 0 && (m + 255) / 256 * 256 - m <= m / 8) {
+    const long long t320x = (long long)((m + 255) / 256) * (n / 320);
+    for (int p = 2; p <= 4; p *= 2)
+      if (t320x * p >= 224 && t320x * p <= 256 && (k / 64) % p == 0 && k / 64 / p >= 32) return {9, p};
+  }
   if (m > 64 && t256 >= 160) {
     // rounds of 256 workgroups times the time of a tile: a 192-row tile does 0.75 of the work
     // of a 256-row one in 0.81 of the time, a 320-row tile 1.25 of it in 1.22 to 1.26 (28,672 gated
@@ -684,7 +694,13 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   // 256 x 128 tiles; 1,024 tokens: 109 against 118)
   if (m > 64 && epilogue == 0 && (k / 64) % 4 == 0 && k / 64 / 4 >= 48 && t256 * 4 >= 192 && t256 * 4 <= 256)
     return {4, 4};
-  if (m > 64 && t256x128 >= 192 && t256x128 <= 256) return {8, 1};
+  // an eighth of a round, of a very deep product, in 8 (8,192 rows at K = 28672, 256 tokens: 122 us against 141
+  // in 4 slices of the 256 x 128 tiles)
+  if (m > 128 && epilogue == 0 && (k / 64) % 8 == 0 && k / 64 / 8 >= 48 && t256 * 8 >= 192 && t256 * 8 <= 256)
+    return {4, 8};
+  // (a gated product, whose K cannot be cut, from 160 such tiles on: 22,016 gated rows, 256 tokens, 172
+  // tiles 64 us against 74 in 344 tiles of 128 x 128)
+  if (m > 64 && t256x128 >= (epilogue == 1 ? 160 : 192) && t256x128 <= 256) return {8, 1};
   if (m > 64 && epilogue == 0) {
     for (int p = 2; p <= 8; p *= 2)
       if (t256x128 * p >= 160 && t256x128 * p <= 256 && (k / 64) % p == 0 && k / 64 / p >= (p == 2 ? 32 : (p == 4 ? (n <= 8192 ? 16 : 32) : 24)))
@@ -699,14 +715,22 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
     if (t192r * 2 >= 160 && t192r * 2 <= 256) return {6, 2};
     if (t256 * 2 >= 160 && t256 * 2 <= 256) return {4, 2};
   }
+  // (at K = 4096 where the 192-row tiles in 2 slices make three quarters of a round or more, up to 768
+  // tokens, beyond which the second slab costs more than that: 12,288 rows, 384 tokens 51 us against 65;
+  // 6,144 rows, 768 tokens 50 against 60)
+  if (m > 64 && m <= 768 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 32 && t192r * 2 >= 192 && t192r * 2 <= 256)
+    return {6, 2};
   if (m > 64 && t192r >= 176 && t192r <= 256) return {6, 1};
   if (m > 64 && (t128 >= 256 || m > 512)) return {5, epilogue ? 1 : k_slices(t128, k, 512, k / (4 * m))};
   // A gated product of at most 64 tokens cannot cut K and streams W from too few workgroups to
   // hide anything (28,672 rows: 224 tiles of 128): tiles of 64 rows, four stages deep, two to a
   // compute unit, up to 24 tokens (17 tokens: 45 us against 50), and K tiles of 128 (256 bytes a
   // row and load) beyond (64 tokens: 49.2 against 50.8).
-  if (m <= 64 && epilogue == 1 && n >= 16384) {
-    if (m <= 24) return {10, 1};
+  // The 64-row tiles only where they are at least one and a half to a compute unit (22,016 gated rows, 344
+  // tiles, 17 tokens: 37 us against 34 with K tiles of 128), and with a deep K the plain 128 x 64 tiles
+  // (57,344 gated rows at K = 8192: 139-147 us against 146-155 at 17 to 64 tokens).
+  if (m <= 64 && epilogue == 1 && n >= 16384 && k < 8192) {
+    if (m <= 24 && (n + 63) / 64 >= 384) return {10, 1};
     if (k % 128 == 0) return {13, 1};
   }
   // At most 64 tokens, no gate: tiles of 128 rows in K slices, or tiles of 64 rows (four stages deep, two
