@@ -370,7 +370,11 @@ static int launch_skinny_u(const GemmTokens& x, const bf16_t* w, void* c, const 
   constexpr int max_waves = (R * MB <= 4) ? 8 : (R * MB <= 8 ? 4 : 3);      // bounds the reduction buffer
   if (k % 128 == 0) {
     const int t = k / 128;
-    int nw = g_tune_waves ? g_tune_waves : ((k >= 8192 || max_waves < 4) ? max_waves : 4);
+    // 8 waves where K is long, or where every compute unit gets one workgroup at most and so needs
+    // more loads in flight of its own (4,096 rows at K = 4096: 8.1-8.3 us against 8.6-9.0 with 4);
+    // 4 where several workgroups share a compute unit (6,144 rows: 10.7 against 11.6 with 8)
+    const long long wgs = (n + 16 * R - 1) / (16 * R);
+    int nw = g_tune_waves ? g_tune_waves : ((k >= 8192 || wgs <= 256 || max_waves < 4) ? max_waves : 4);
     if (nw > max_waves) nw = max_waves;
     if (nw > t) nw = t;
     return launch_skinny<MB, R, 1, true, EPI, TO, SCALED>(x, w, c, after, m, n, k, nw, 0, s);
@@ -397,7 +401,9 @@ static int dispatch_skinny(const GemmTokens& x, const bf16_t* w, void* c, const 
   // compute units more evenly: the time goes with the rows that the busiest compute unit gets, at
   // a price per row that falls with R (about 15 % / R).  57344 rows at K = 8192: R = 4 gives 896
   // workgroups, 4 on some compute units and 3 on others, 194 us; R = 2 gives every one 7: 175 us.
-  // 10240 rows at K = 8192 with one token: R = 1 35 us, R = 2 42.
+  // 10240 rows at K = 8192 with one token: R = 1 35 us, R = 2 42; R = 4 takes 31 us by itself (160
+  // workgroups), but the decode step of that shape is no faster with it (+0.3 % at batch 1, +0.5 % at
+  // 8, -1.1 % at 16, each the mean of four runs in alternating order), so it is not taken.
   int r = 1;
   if (k >= 8192) {
     double best = 0.0;
