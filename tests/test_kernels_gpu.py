@@ -679,6 +679,42 @@ def test_gemm_terms_and_the_norm_that_adds_them(lib, m, n, k):
             assert torch.equal(xa, x0 + whole)
 
 
+@pytest.mark.parametrize("m,n,k,gated,min_terms", [
+    (512, 10240, 8192, False, 4),      # 320-row tiles in 4 K slices
+    (192, 8192, 28672, False, 8),      # 256 x 256 tiles in 8 slices of a very deep K
+    (1536, 4096, 14336, False, 2),     # 256 x 256 tiles in 2 slices
+    (384, 12288, 4096, False, 2),      # 192-row tiles in 2 slices at K = 4096
+    (64, 4096, 11008, False, 4),       # 64-row tiles where 8 slices do not divide K
+    (48, 4096, 4096, False, 4),        # 64-row tiles in half as many slices
+    (96, 57344, 8192, True, 1),        # 256 x 128 tiles among the large ones
+    (256, 22016, 4096, True, 1),       # 172 tiles of 256 x 128, gated
+    (24, 22016, 4096, True, 1),        # gated, few tokens, K tiles of 128
+])
+def test_products_of_the_model_shapes_the_tile_planner_has_rules_for(lib, m, n, k, gated, min_terms):
+    """The sizes for which the planner picks a tile or a number of K slices by a rule of its
+    own, with W stored fragment-major as the engine stores it, against a float32 product."""
+    from helpers import fragment_major
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16().to(DEV)
+    wf = fragment_major(w)
+    if gated:
+        out = torch.full((m, n // 2), float("nan"), device=DEV, dtype=torch.bfloat16)
+        lib.gemm_bf16(a, wf, out, 1, w_frag=True)
+        wr = w.float().view(n // 32, 2, 16, k)
+        gate = a.float() @ wr[:, 0].reshape(n // 2, k).T
+        up = a.float() @ wr[:, 1].reshape(n // 2, k).T
+        want = torch.nn.functional.silu(gate) * up
+        assert _rel(out, want) < 1e-2
+        return
+    terms = lib.gemm_bf16_terms(a, wf, w_frag=True)
+    assert terms.shape[0] >= min_terms and terms.shape[1:] == (m, n)
+    want = a.float() @ w.float().T
+    assert _rel(terms.sum(0), want) < 2e-3
+    rows = lib.gemm_bf16_terms(a, w)                     # the same product with W as rows: the same bits
+    assert torch.equal(rows, terms)
+
+
 def test_gemm_bf16_few_refuses_other_sizes(lib):
     from rbitnet_amd.errors import KernelError
     assert not lib.gemm_bf16_few_ok(17, 64, 64)
