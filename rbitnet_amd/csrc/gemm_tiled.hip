@@ -667,6 +667,13 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
     // against 414).
     const long long t128t = (long long)((m + 127) / 128) * ((n + 255) / 256);
     const long long cost128t = (t128t + 255) / 256 * 650;
+    // A very deep product in 2 K slices of the 256 x 256 tiles where that fills the last round better (8,192
+    // rows at K = 28672, 3,072 tokens: 384 tiles, one and a half rounds that take the time of two; 768 half
+    // tiles make three rounds of half the time: 1,125 us against 1,300, and 40 us for the second slab).
+    if (epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 128) {
+      const long long cost256x2 = (2 * t256 + 255) / 256 * 500 + 60;
+      if (cost256x2 < cost256 && cost256x2 < cost192 && cost256x2 < cost320 && cost256x2 < cost128t) return {4, 2};
+    }
     if (cost128t < cost256 && cost128t < cost192 && cost128t < cost320) return {8, 1};
     if (cost320 < cost256 && cost320 < cost192) return {9, 1};
     return {cost192 < cost256 ? 6 : 4, 1};
