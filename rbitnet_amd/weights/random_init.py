@@ -25,7 +25,6 @@ from __future__ import annotations
 
 import hashlib
 import json
-import math
 import os
 from collections.abc import Mapping
 from typing import Any, Dict, Iterator, Tuple

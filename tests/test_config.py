@@ -4,7 +4,6 @@ import json
 
 import pytest
 
-import rbitnet_amd
 from rbitnet_amd.config import LlamaConfig, load_config, registered_architectures
 from rbitnet_amd.errors import ConfigError
 

@@ -7,7 +7,6 @@ import struct
 import pytest
 import torch
 
-import rbitnet_amd
 from rbitnet_amd.config import LlamaConfig, load_config
 from rbitnet_amd.engine.model import expected_tensors
 from rbitnet_amd.errors import WeightError
