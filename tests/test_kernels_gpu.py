@@ -715,6 +715,39 @@ def test_products_of_the_model_shapes_the_tile_planner_has_rules_for(lib, m, n, 
     assert torch.equal(rows, terms)
 
 
+@pytest.mark.parametrize("cfg", [4, 5, 6, 7, 8, 9, 10, 13])
+def test_every_tile_of_the_direct_to_lds_product_at_sizes_that_fill_none(lib, cfg):
+    """The planner picks a tile by the product's sizes, so sizes of a test reach only some of the
+    tiles: here each is forced in turn (the hook that measurements use), with 1, 2 and 4 K slices,
+    for token and row counts that fill no tile (rows a multiple of 16 only, as fragment-major W
+    asks), W as rows and fragment-major, plain and gated."""
+    from helpers import fragment_major
+    k = 1024
+    try:
+        for m, n in ((33, 992), (200, 592), (300, 1376)):
+            g = torch.Generator().manual_seed(cfg * 1000 + m)
+            a = torch.randn(m, k, generator=g).bfloat16().to(DEV)
+            w = (torch.randn(n, k, generator=g) * 0.05).bfloat16().to(DEV)
+            wf = fragment_major(w)
+            want = a.float() @ w.float().T
+            for parts in (1, 2, 4):
+                lib._lib.rb_tune_tiles(cfg, parts)
+                terms = lib.gemm_bf16_terms(a, wf, w_frag=True)
+                assert terms.shape == (parts, m, n), (cfg, parts, tuple(terms.shape))
+                assert _rel(terms.sum(0), want) < 2e-3, (cfg, m, n, parts)
+                assert torch.equal(lib.gemm_bf16_terms(a, w), terms), (cfg, m, n, parts)
+            lib._lib.rb_tune_tiles(cfg, 1)
+            if n % 32 == 0:
+                out = torch.full((m, n // 2), float("nan"), device=DEV, dtype=torch.bfloat16)
+                lib.gemm_bf16(a, wf, out, 1, w_frag=True)
+                wr = w.float().view(n // 32, 2, 16, k)
+                gate = a.float() @ wr[:, 0].reshape(n // 2, k).T
+                up = a.float() @ wr[:, 1].reshape(n // 2, k).T
+                assert _rel(out, torch.nn.functional.silu(gate) * up) < 1e-2, (cfg, m, n)
+    finally:
+        lib._lib.rb_tune_tiles(0, 0)
+
+
 def test_gemm_bf16_few_refuses_other_sizes(lib):
     from rbitnet_amd.errors import KernelError
     assert not lib.gemm_bf16_few_ok(17, 64, 64)
