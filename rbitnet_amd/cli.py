@@ -224,6 +224,11 @@ def main(argv: Optional[List[str]] = None) -> int:
     except RbitnetError as e:
         print(f"error: {e}", file=sys.stderr)
         return 1
+    except BrokenPipeError:
+        # the reader of our output has gone (`... | head`): not an error of ours; point stdout at
+        # /dev/null so that the interpreter's flush at exit does not complain either
+        os.dup2(os.open(os.devnull, os.O_WRONLY), sys.stdout.fileno())
+        return 0
     except OSError as e:
         print(f"error: IO error: {e}", file=sys.stderr)
         return 1
