@@ -173,6 +173,60 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_head: int, n_
     return out
 
 
+def rope_rows(x: torch.Tensor, n_heads: int, inv_freq: torch.Tensor, style: str = "interleaved",
+              first_pos: int = 0) -> torch.Tensor:
+    """`rope` for every row and head of x [T, n_heads * D] at once (row t at position first_pos + t):
+    the same pairs, angles and signs written with whole-tensor operations, for sequences of hundreds
+    of tokens at the widths of real models.  tests/test_plain.py holds it equal to `rope`."""
+    t_len = x.shape[0]
+    d = x.shape[1] // n_heads
+    half = d // 2
+    pos = torch.arange(first_pos, first_pos + t_len, dtype=torch.float64)
+    a = pos[:, None] * inv_freq.to(torch.float64)[None, :]                # [T, D/2]
+    c = torch.cos(a).to(device=x.device, dtype=x.dtype)[:, None, :]
+    s = torch.sin(a).to(device=x.device, dtype=x.dtype)[:, None, :]
+    v = x.reshape(t_len, n_heads, d)
+    if style == "interleaved":
+        x0, x1 = v[..., 0::2], v[..., 1::2]
+    elif style == "half":
+        x0, x1 = v[..., :half], v[..., half:]
+    else:
+        raise ValueError(style)
+    y0 = x0 * c - x1 * s
+    y1 = x0 * s + x1 * c
+    out = torch.empty_like(v)
+    if style == "interleaved":
+        out[..., 0::2], out[..., 1::2] = y0, y1
+    else:
+        out[..., :half], out[..., half:] = y0, y1
+    return out.reshape(t_len, n_heads * d)
+
+
+def attention_rows(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, n_head: int, n_kv: int,
+                   window: int | None = None, round_weights=None) -> torch.Tensor:
+    """`attention` with one [T, T] score matrix per head in place of the loop over positions: the
+    same scale, mask, maximum, sum and weighting.  tests/test_plain.py holds it equal to `attention`."""
+    t_len = q.shape[0]
+    d = q.shape[1] // n_head
+    n_rep = n_head // n_kv
+    scale = 1.0 / math.sqrt(d)
+    pos = torch.arange(t_len, device=q.device)
+    seen = pos[None, :] <= pos[:, None]
+    if window is not None:
+        seen = seen & (pos[:, None] - pos[None, :] < window)
+    out = torch.zeros(t_len, n_head * d, dtype=q.dtype, device=q.device)
+    for qh in range(n_head):
+        kvh = qh // n_rep
+        scores = (q[:, qh * d:(qh + 1) * d] @ k[:, kvh * d:(kvh + 1) * d].T) * scale
+        scores = scores.masked_fill(~seen, -math.inf)
+        z = torch.exp(scores - scores.max(dim=1, keepdim=True).values)
+        total = z.sum(dim=1, keepdim=True)
+        if round_weights is not None:
+            z = round_weights(z)
+        out[:, qh * d:(qh + 1) * d] = (z / total) @ v[:, kvh * d:(kvh + 1) * d]
+    return out
+
+
 def swiglu(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
     """down( silu(gate h) * (up h) ).  model.rs:297-303."""
     g = silu(linear(h, w_gate))
@@ -185,14 +239,18 @@ def swiglu(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: to
 class PlainLlama:
     """config.json + tensors by name -> logits of whole sequences."""
 
-    def __init__(self, config: dict, tensors: dict, dtype=torch.float64, device="cpu", round_bf16: bool = False):
-        """round_bf16: round to bfloat16 wherever an engine that computes in bfloat16 stores a
+    def __init__(self, config: dict, tensors: dict, dtype=torch.float64, device="cpu", round_bf16: bool = False,
+                 rows_at_once: bool = False):
+        """rows_at_once: rotation, attention and matrix products through `rope_rows`, `attention_rows`
+        and one matrix product per call (the forms for long sequences at real widths).
+        round_bf16: round to bfloat16 wherever an engine that computes in bfloat16 stores a
         value in that type (normalised rows, rotated q and k, v, the weights of the values, the
         attention output, the gated activation), everything else as before.  The distance of
         that from the exact logits is what such an engine cannot avoid; its distance from an
         engine's logits is what the engine adds."""
         c = config
         self.round_bf16 = round_bf16
+        self.rows_at_once = rows_at_once
         self.dtype = dtype
         self.device = device        # where the sums run; the element-by-element rotation stays on the host
         self.n_embd = int(c["hidden_size"])
@@ -215,12 +273,13 @@ class PlainLlama:
         self.w = {k: v.to(device=device, dtype=dtype) for k, v in tensors.items()}
 
     @classmethod
-    def from_folder(cls, folder: str, dtype=torch.float64, device="cpu", round_bf16: bool = False) -> "PlainLlama":
+    def from_folder(cls, folder: str, dtype=torch.float64, device="cpu", round_bf16: bool = False,
+                    rows_at_once: bool = False) -> "PlainLlama":
         from safetensors.torch import load_file
         with open(os.path.join(folder, "config.json")) as f:
             config = json.load(f)
         tensors = load_file(os.path.join(folder, "model.safetensors"))
-        return cls(config, tensors, dtype, device, round_bf16)
+        return cls(config, tensors, dtype, device, round_bf16, rows_at_once)
 
     def _r(self, t: torch.Tensor) -> torch.Tensor:
         return t.to(torch.bfloat16).to(t.dtype) if self.round_bf16 else t
@@ -231,27 +290,36 @@ class PlainLlama:
         p = f"model.layers.{il}."
         w = self.w
         d = self.head_dim
+        lin = self._linear
         h = self._r(rmsnorm(x, w[p + "input_layernorm.weight"], self.eps))
-        q = linear(h, w[p + "self_attn.q_proj.weight"])
-        k = linear(h, w[p + "self_attn.k_proj.weight"])
-        v = linear(h, w[p + "self_attn.v_proj.weight"])
-        q, k = q.cpu(), k.cpu()
-        for pos in range(x.shape[0]):
-            for hh in range(self.n_head):
-                q[pos, hh * d:(hh + 1) * d] = rope(q[pos, hh * d:(hh + 1) * d], pos, self.inv_freq, self.style)
-            for hh in range(self.n_kv):
-                k[pos, hh * d:(hh + 1) * d] = rope(k[pos, hh * d:(hh + 1) * d], pos, self.inv_freq, self.style)
+        q = lin(h, w[p + "self_attn.q_proj.weight"])
+        k = lin(h, w[p + "self_attn.k_proj.weight"])
+        v = lin(h, w[p + "self_attn.v_proj.weight"])
+        if self.rows_at_once:
+            q = rope_rows(q, self.n_head, self.inv_freq, self.style)
+            k = rope_rows(k, self.n_kv, self.inv_freq, self.style)
+        else:
+            q, k = q.cpu(), k.cpu()
+            for pos in range(x.shape[0]):
+                for hh in range(self.n_head):
+                    q[pos, hh * d:(hh + 1) * d] = rope(q[pos, hh * d:(hh + 1) * d], pos, self.inv_freq, self.style)
+                for hh in range(self.n_kv):
+                    k[pos, hh * d:(hh + 1) * d] = rope(k[pos, hh * d:(hh + 1) * d], pos, self.inv_freq, self.style)
         q, k, v = self._r(q.to(x.device)), self._r(k.to(x.device)), self._r(v)
-        a = self._r(attention(q, k, v, self.n_head, self.n_kv, self.window,
-                              round_weights=self._r if self.round_bf16 else None))
-        x = x + linear(a, w[p + "self_attn.o_proj.weight"])
+        attend = attention_rows if self.rows_at_once else attention
+        a = self._r(attend(q, k, v, self.n_head, self.n_kv, self.window,
+                           round_weights=self._r if self.round_bf16 else None))
+        x = x + lin(a, w[p + "self_attn.o_proj.weight"])
         h2 = self._r(rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps))
-        if self.round_bf16:
-            t = self._r(silu(linear(h2, w[p + "mlp.gate_proj.weight"])) * linear(h2, w[p + "mlp.up_proj.weight"]))
-            return x + linear(t, w[p + "mlp.down_proj.weight"])
+        if self.round_bf16 or self.rows_at_once:
+            t = self._r(silu(lin(h2, w[p + "mlp.gate_proj.weight"])) * lin(h2, w[p + "mlp.up_proj.weight"]))
+            return x + lin(t, w[p + "mlp.down_proj.weight"])
         x = x + swiglu(h2, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                        w[p + "mlp.down_proj.weight"])
         return x
+
+    def _linear(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        return x @ w.T if self.rows_at_once else linear(x, w)
 
     def hidden(self, tokens) -> torch.Tensor:
         x = embedding(self.w["model.embed_tokens.weight"], tokens)
@@ -259,12 +327,15 @@ class PlainLlama:
             x = self.layer(x, il)
         return x
 
-    def logits(self, tokens) -> torch.Tensor:
-        """Logits [T, V] at every position of one sequence.  model.rs:229-315."""
+    def logits(self, tokens, last: int | None = None) -> torch.Tensor:
+        """Logits [T, V] at every position of one sequence (`last`: at its last that many
+        positions only).  model.rs:229-315."""
         x = self.hidden(tokens)
+        if last is not None:
+            x = x[-last:]
         xn = self._r(rmsnorm(x, self.w["model.norm.weight"], self.eps))
         head = self.w["model.embed_tokens.weight"] if self.tied else self.w["lm_head.weight"]
-        return linear(xn, head)
+        return self._linear(xn, head)
 
 
 # --------------------------------------------------------------------------- sampling

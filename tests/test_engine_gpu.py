@@ -92,6 +92,36 @@ def test_unequal_batches_with_slot_reuse(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_prompts_in_pieces_for_several_sequences_at_once(name, dtype):
+    """Steps that bring several tokens per sequence on top of pasts that differ per sequence (a
+    prompt fed in pieces, batched): pieces that end inside a page, at its edge and beyond it, a
+    sequence that brings one token while its neighbours bring many."""
+    lengths = [130, 64, 75]
+    cuts = [[60, 5, 64], [4, 59, 1], [66, 0, 9]]            # tokens per sequence and step; 0: it sits the step out
+    reqs = [tokens_for(name, n, 60 + i) for i, n in enumerate(lengths)]
+    eng = _engine(name, dtype, max_batch=3, max_tokens=64 * 5)
+    for g in eng.cache.kv_groups:
+        g.k.fill_(float("nan"))
+        g.v.fill_(float("nan"))
+    slots = [eng.alloc_slot() for _ in reqs]
+    done = [0] * len(reqs)
+    got = [[] for _ in reqs]
+    for cut in cuts:
+        live = [i for i, n in enumerate(cut) if n]
+        logits = eng.step([(slots[i], reqs[i][done[i]:done[i] + cut[i]]) for i in live], "all")
+        off = 0
+        for i in live:
+            got[i].append(logits[off:off + cut[i]])
+            off += cut[i]
+            done[i] += cut[i]
+    assert done == lengths
+    for i, r in enumerate(reqs):
+        err = max_err(torch.cat(got[i]), plain_logits(name, tuple(r)))
+        assert err < TOL[dtype], f"{name} {dtype} request {i}: {err}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_batch_that_shrinks_from_20_sequences_to_8(name, dtype):
     """Steps of more than 16 tokens and of at most 16 run different kernels (with few tokens the

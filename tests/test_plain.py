@@ -247,3 +247,28 @@ def test_sampling():
     for i in range(4000):
         hist[P.sample_token(z, 1.0, (i + 0.5) / 4000)] += 1
     assert abs(hist[0] / 4000 - 0.25) < 0.01
+
+
+def test_forms_for_long_sequences_equal_the_loops():
+    """`rope_rows`, `attention_rows` and the model's rows_at_once mode are the element-by-element
+    functions written with whole-tensor operations: equal to them up to the order of float64 sums."""
+    t_len, hq, hk, d = 9, 6, 2, 8
+    inv = P.rope_inv_freq(d, 10000.0, None)
+    x = torch.randn(t_len, hq * d, dtype=D64)
+    for style in ("interleaved", "half"):
+        want = torch.stack([torch.cat([P.rope(x[t, h * d:(h + 1) * d], t + 3, inv, style) for h in range(hq)])
+                            for t in range(t_len)])
+        assert torch.allclose(P.rope_rows(x, hq, inv, style, first_pos=3), want, atol=1e-14)
+    q, k, v = x, torch.randn(t_len, hk * d, dtype=D64), torch.randn(t_len, hk * d, dtype=D64)
+    for window in (None, 4):
+        assert torch.allclose(P.attention_rows(q, k, v, hq, hk, window), P.attention(q, k, v, hq, hk, window),
+                              atol=1e-13)
+    rounded = lambda t: t.to(torch.bfloat16).to(t.dtype)
+    assert torch.allclose(P.attention_rows(q, k, v, hq, hk, None, rounded),
+                          P.attention(q, k, v, hq, hk, None, round_weights=rounded), atol=1e-13)
+    for name in ("A", "B"):
+        folder = model_folder(name)
+        toks = [3, 200, 17, 5, 5, 90, 41, 7, 250, 0, 13]
+        slow, fast = P.PlainLlama.from_folder(folder), P.PlainLlama.from_folder(folder, rows_at_once=True)
+        assert torch.allclose(fast.logits(toks), slow.logits(toks), atol=1e-12)
+        assert torch.allclose(fast.logits(toks, last=3), fast.logits(toks)[-3:], atol=1e-13)
