@@ -43,8 +43,19 @@ LLAMA31_70B = {
     "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
                      "original_max_position_embeddings": 8192},
 }
+# widths that no rule of the product planners was fitted to (measured as a check of those rules)
+def _other(hidden, ff, heads, kv_heads, head_dim, layers, vocab=128256):
+    return {"architectures": ["LlamaForCausalLM"], "hidden_size": hidden, "num_hidden_layers": layers,
+            "num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": head_dim,
+            "intermediate_size": ff, "vocab_size": vocab, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
+            "max_position_embeddings": 8192, "tie_word_embeddings": False}
+
+
 MODELS = {"llama3_8b": ("Llama-3-8B shape", LLAMA3_8B), "llama2_7b": ("Llama-2-7B shape", LLAMA2_7B),
-          "llama31_70b": ("Llama-3.1-70B shape", LLAMA31_70B)}
+          "llama31_70b": ("Llama-3.1-70B shape", LLAMA31_70B),
+          "w2048": ("hidden 2048, 32 heads of 64 on 8", _other(2048, 8192, 32, 8, 64, 16)),
+          "w3072": ("hidden 3072, 24 heads of 128 on 8", _other(3072, 8192, 24, 8, 128, 28)),
+          "w5120": ("hidden 5120, 40 heads of 128 on 40", _other(5120, 13824, 40, 40, 128, 40, vocab=32000))}
 PROMPT_LEN = 512
 NEW_TOKENS = 256
 PREFILL_TOKENS = 2048
@@ -148,8 +159,13 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--points", default="1,64", help="batch sizes of the extra decode points")
-    ap.add_argument("--model", default="llama3_8b", choices=sorted(MODELS),
-                    help="shape to measure (default: the baseline's configs[2])")
+    ap.add_argument("--model", default="llama3_8b",
+                    help=f"shape to measure, one of {', '.join(sorted(MODELS))} (default: the baseline's configs[2]); "
+                         "with --planner-sweep several, separated by commas")
+    ap.add_argument("--planner-sweep", action="store_true",
+                    help="no benchmark: time every product of the named shapes with the planner's choice and with "
+                         "every choice forced (see planner_check.py)")
+    ap.add_argument("--tokens", default="1,8,64,512,2048", help="token counts of --planner-sweep")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="length of the one prompt whose prefill is timed")
     ap.add_argument("--prompt-len", default=str(PROMPT_LEN),
@@ -158,6 +174,17 @@ def main(argv=None) -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (this library has no multi-GPU path); --gpus {args.gpus} is not run")
         return 2
+
+    names = [v for v in args.model.split(",") if v]
+    for name in names:
+        if name not in MODELS:
+            ap.error(f"unknown --model {name!r}; one of {', '.join(sorted(MODELS))}")
+    if args.planner_sweep:
+        from .planner_check import sweep
+        sweep([(MODELS[n][0], MODELS[n][1]) for n in names], [int(v) for v in args.tokens.split(",") if v])
+        return 0
+    if len(names) != 1:
+        ap.error("one --model at a time")
 
     import torch
     from .engine import Engine
@@ -190,7 +217,7 @@ def main(argv=None) -> int:
     value = args.batch * args.steps / dt
 
     hk = cfg["num_key_value_heads"]
-    d = cfg["hidden_size"] // cfg["num_attention_heads"]
+    d = cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_attention_heads"]
     esize = 2 if args.dtype == "bf16" else 4
     kv_bytes_per_token = 2 * hk * d * esize * layers
     step_bytes = engine.model.weight_bytes() + args.batch * ctx_mean * kv_bytes_per_token

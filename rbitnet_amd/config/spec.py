@@ -11,6 +11,11 @@ and the prefix under which its tensors are stored.  `ModelSpec.schedule` is the
 order in which layers run: a list of indices into `layers`, which may name a
 layer twice.  A mixer whose parameters hold `cache_from = j` keeps no cache of
 its own and reads the one layer `j` wrote.
+
+The two ends of a model are parts too: `embedding` (token ids -> stream) and `head`
+(stream -> logits).  A spec that does not name them gets the plain ones, built from
+`embedding_name`, `final_norm`, `final_norm_name` and `head_name`: a table whose rows are
+gathered, and a norm followed by a matrix (the table again when `head_name` is None).
 """
 from __future__ import annotations
 
@@ -50,18 +55,31 @@ class ModelSpec:
     hidden_size: int
     vocab_size: int
     max_positions: int
-    embedding_name: str
     layers: List[LayerSpec]
-    final_norm: PartSpec
-    final_norm_name: str
-    head_name: Optional[str]          # None: the head is the embedding table (tied)
+    # the plain ends, by their tensors (see the module's text); a spec that names `embedding` and `head`
+    # itself needs none of the four
+    embedding_name: Optional[str] = None
+    final_norm: Optional[PartSpec] = None
+    final_norm_name: Optional[str] = None
+    head_name: Optional[str] = None          # None: the head is the embedding table (tied)
     schedule: List[int] = field(default_factory=list)
     stop_token_ids: List[int] = field(default_factory=list)
     bos_token_id: Optional[int] = None
     # tensors that a weight file may hold without the model reading them
     optional_tensors: List[str] = field(default_factory=list)
+    embedding: Optional[PartSpec] = None
+    head: Optional[PartSpec] = None
 
     def __post_init__(self) -> None:
+        if self.embedding is None:
+            if self.embedding_name is None:
+                raise ValueError("a model needs an embedding: name the part, or the table's tensor")
+            self.embedding = PartSpec("table", {"name": self.embedding_name, "vocab_size": self.vocab_size})
+        if self.head is None:
+            if self.final_norm is None or self.final_norm_name is None:
+                raise ValueError("a model needs a head: name the part, or the final norm and its tensor")
+            self.head = PartSpec("linear", {"norm": self.final_norm, "norm_name": self.final_norm_name,
+                                            "name": self.head_name, "vocab_size": self.vocab_size})
         if not self.schedule:
             self.schedule = list(range(len(self.layers)))
         for i in self.schedule:

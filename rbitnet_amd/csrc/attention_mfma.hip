@@ -46,14 +46,15 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
   const int groups_per_kv = group / gw;
   // Which block of queries and which heads.  The blocks of late queries have the most keys:
   // they are started first (block index 0 is the last block), and the short ones fill the
-  // compute units that finish early.  `paired`: the workgroups of a sequence, two of which fit
-  // a compute unit, are all resident at once (at most 512 of them); then the first 256 are the
-  // heaviest in falling order and the rest the lightest in rising order, so that the two that
-  // share a compute unit have about the same work together everywhere.
+  // compute units that finish early.  `paired` (the number of compute units, or 0): the workgroups
+  // of a sequence, two of which fit a compute unit, are all resident at once (at most two per
+  // compute unit); then the first `paired` are the heaviest in falling order and the rest the
+  // lightest in rising order, so that the two that share a compute unit have about the same work
+  // together everywhere.
   int bx = blockIdx.x, by = blockIdx.y;
   if (paired) {
     const int n = gridDim.x * gridDim.y, at = blockIdx.x + gridDim.x * blockIdx.y;
-    const int rank = at < 256 ? at : n - 1 - (at - 256);
+    const int rank = at < paired ? at : n - 1 - (at - paired);
     by = rank % gridDim.y;
     bx = rank / gridDim.y;
   }
@@ -324,7 +325,8 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
   if (g_prefill_waves) nw = g_prefill_waves;
   const int q_per_wg = 32 * (nw / gw);
   dim3 grid((max_q_len + q_per_wg - 1) / q_per_wg, n_kv_heads * (group / gw), n_seqs);
-  const int paired = (nw == 4 && g_prefill_paired && grid.x * grid.y > 256 && grid.x * grid.y <= 512) ? 1 : 0;
+  const int cus = rb_compute_units();
+  const int paired = (nw == 4 && g_prefill_paired && (int)(grid.x * grid.y) > cus && (int)(grid.x * grid.y) <= 2 * cus) ? cus : 0;
   RB_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "rb_attention_prefill_bf16: batch or head count too large");
   hipStream_t s = (hipStream_t)stream;
   const float sl2 = scale * LOG2E;
@@ -1028,13 +1030,14 @@ extern "C" void rb_tune_decode_waves(int nw) { g_decode_waves = nw; }      // ex
 template <int D, bool FUSED>
 static int launch_decode_mfma(const DecodeArgs& a, hipStream_t s) {
   const long long wgs = (long long)a.n_splits * a.n_kv * a.n_seqs;
-  const int nw = g_decode_waves ? g_decode_waves : (wgs <= 256 && a.n_splits == 1 ? 8 : 4);
+  const int cus = rb_compute_units();
+  const int nw = g_decode_waves ? g_decode_waves : (wgs <= cus && a.n_splits == 1 ? 8 : 4);
   // Pages past the caches.  V when the batch is large enough for the caches to matter (32 sequences x
   // kv heads and more: batch 64 1.9 % of the step, batch 8 0.8 %; with a single sequence the plain loads
   // are 1.2 % faster).  The keys as well where the launch is large (512 workgroups and more: batch 64
   // at 8,192 keys 4.7 % of the step, at 530 keys 1.9 %); in small launches, which wait for their first
   // page rather than for bandwidth, they lose (batch 8 at 530 keys: 0.9 %).
-  const int once = (long long)a.n_kv * a.n_seqs < 32 ? 0 : (wgs >= 512 ? 2 : 1);
+  const int once = (long long)a.n_kv * a.n_seqs < cus / 8 ? 0 : (wgs >= 2 * cus ? 2 : 1);
   if (nw == 8) {
     if (once == 0) return launch_decode_mfma_nw<D, 8, FUSED, 0>(a, s);
     if (once == 1) return launch_decode_mfma_nw<D, 8, FUSED, 1>(a, s);

@@ -29,6 +29,12 @@ void rb_set_error(const char* fmt, ...);
 
 enum RbDtype { RB_F32 = 0, RB_BF16 = 1 };
 
+// ---------------------------------------------------------------- the machine
+// Compute units of the current device (asked of the runtime once per device): what one round
+// of workgroups is.  Every choice of a tile, a number of K slices or of splits that depends on
+// how a grid fills the GPU is an expression of this number, not of the 256 of an MI355X.
+int rb_compute_units(void);
+
 // ---------------------------------------------------------------- bfloat16 storage
 struct bf16_t {
   uint16_t bits;

@@ -18,6 +18,22 @@ extern "C" const char* rb_last_error(void) { return g_error; }
 extern "C" int rb_version(void) { return 1; }
 extern "C" int rb_page_size(void) { return RB_PAGE; }
 
+// ---------------------------------------------------------------- the machine
+static int g_tune_cus = 0;
+extern "C" void rb_tune_compute_units(int n) { g_tune_cus = n; }      // tests and experiments; 0 = the device's own
+int rb_compute_units(void) {
+  if (g_tune_cus > 0) return g_tune_cus;
+  static int known[64];                 // per device, 0 = not asked yet (a race writes the same number twice)
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (known[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    known[dev] = n;
+  }
+  return known[dev];
+}
+
 // ---------------------------------------------------------------- embedding
 // Reference: x[j] = token_embd[j + tok * n_embd] (llama/model.rs:229-232).
 template <typename T>

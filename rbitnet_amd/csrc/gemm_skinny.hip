@@ -374,7 +374,7 @@ static int launch_skinny_u(const GemmTokens& x, const bf16_t* w, void* c, const 
     // more loads in flight of its own (4,096 rows at K = 4096: 8.1-8.3 us against 8.6-9.0 with 4);
     // 4 where several workgroups share a compute unit (6,144 rows: 10.7 against 11.6 with 8)
     const long long wgs = (n + 16 * R - 1) / (16 * R);
-    int nw = g_tune_waves ? g_tune_waves : ((k >= 8192 || wgs <= 256 || max_waves < 4) ? max_waves : 4);
+    int nw = g_tune_waves ? g_tune_waves : ((k >= 8192 || wgs <= rb_compute_units() || max_waves < 4) ? max_waves : 4);
     if (nw > max_waves) nw = max_waves;
     if (nw > t) nw = t;
     return launch_skinny<MB, R, 1, true, EPI, TO, SCALED>(x, w, c, after, m, n, k, nw, 0, s);
@@ -407,9 +407,10 @@ static int dispatch_skinny(const GemmTokens& x, const bf16_t* w, void* c, const 
   int r = 1;
   if (k >= 8192) {
     double best = 0.0;
+    const long long cus = rb_compute_units();
     for (int cand = (EPI == 1 ? 2 : 1); cand <= 4; cand *= 2) {
       const long long wgs = (n + 16 * cand - 1) / (16 * cand);
-      const double cost = (double)((wgs + 255) / 256 * 16 * cand) * (1.0 + 0.15 / cand);
+      const double cost = (double)((wgs + cus - 1) / cus * 16 * cand) * (1.0 + 0.15 / cand);
       if (best == 0.0 || cost <= best) {
         best = cost;
         r = cand;
@@ -633,7 +634,8 @@ static int launch_resident(const GemmTokens& x, const bf16_t* w, void* c, const 
   // than 16 (measured: 22016 rows in 230 workgroups of 6 tiles take 35 us, in 344 of 4, which
   // come in two rounds, 44 us; 12288 rows 20 us in 256 workgroups, 31 us in 384; the 128256
   // rows of an output layer are as fast in 501 workgroups of 16 tiles as in 251 of 32)
-  int tiles = g_res_tiles ? g_res_tiles : (n_tiles + 255) / 256;
+  const int cus = rb_compute_units();
+  int tiles = g_res_tiles ? g_res_tiles : (n_tiles + cus - 1) / cus;
   if (!g_res_tiles && tiles > 16) tiles = 16;
   if (EPI == 1 && (tiles & 1)) tiles += 1;
   const size_t lds = ((size_t)2 * (n_waves - 1) * MB * 4 * 64 + (SCALED ? n_waves * MB * 16 : 0)) * sizeof(float);

@@ -617,7 +617,7 @@ extern "C" void rb_tune_tiles(int cfg, int parts) {       // experiments only; 0
 // The most slices that keep the workgroups within `slots`, the slices at least 4 tiles deep
 // and equal, and their number within `cap` (every slice writes and re-reads an [M, N] slab,
 // 8 bytes per element, against W's 2 N K bytes).
-static int k_slices(long long tiles, int k, int slots, int cap) {
+static int k_slices(long long tiles, int k, long long slots, int cap) {
   const int kt = k / 64;
   if (cap > 16) cap = 16;
   int best = 1;
@@ -627,13 +627,17 @@ static int k_slices(long long tiles, int k, int slots, int cap) {
 }
 
 static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
+  // One round: a workgroup on every compute unit.  The thresholds below are the measured ones of a GPU
+  // with 256 compute units, kept as fractions of a round (5/8, 11/16, 3/4, 25/32, 7/8, 1, 3/2, 2).
+  const long long R = rb_compute_units();
+  const auto rounds = [R](long long tiles) { return (tiles + R - 1) / R; };
   const bool dma = k % 64 == 0 && (long long)k * 512 < (1LL << 32);
   const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
   if (!dma) {
     if (m <= 64) return {0, 1};
     const long long t256x128 = (long long)((m + 127) / 128) * ((n + 255) / 256);
     if (g_tile_cfg >= 1 && g_tile_cfg <= 3) return {g_tile_cfg, 1};
-    return {t256 >= 160 ? 3 : (k >= 8192 && t256x128 >= 200 ? 2 : 1), 1};
+    return {t256 >= R * 5 / 8 ? 3 : (k >= 8192 && t256x128 >= R * 25 / 32 ? 2 : 1), 1};
   }
   if (m <= 16) return {0, 1};
   if (g_tile_cfg >= 4) {
@@ -650,9 +654,9 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   if (m > 64 && epilogue == 0 && n % 320 == 0 && (m + 255) / 256 * 256 - m <= m / 8) {
     const long long t320x = (long long)((m + 255) / 256) * (n / 320);
     for (int p = 2; p <= 4; p *= 2)
-      if (t320x * p >= 224 && t320x * p <= 256 && (k / 64) % p == 0 && k / 64 / p >= 32) return {9, p};
+      if (t320x * p >= R * 7 / 8 && t320x * p <= R && (k / 64) % p == 0 && k / 64 / p >= 32) return {9, p};
   }
-  if (m > 64 && t256 >= 160) {
+  if (m > 64 && t256 >= R * 5 / 8) {
     // rounds of 256 workgroups times the time of a tile: a 192-row tile does 0.75 of the work
     // of a 256-row one in 0.81 of the time, a 320-row tile 1.25 of it in 1.22 to 1.26 (28,672 gated
     // rows by 2,048 tokens: 896 tiles of 256 rows, 3.5 rounds, 475 us; 720 of 320 rows, under 3
@@ -660,18 +664,17 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
     // 4,096 tokens in steps of 128, and for 6,144 and 4,096 rows: within 2 % everywhere.
     const long long t192 = (long long)((m + 255) / 256) * ((n + 191) / 192);
     const long long t320 = (long long)((m + 255) / 256) * ((n + 319) / 320);
-    const long long cost256 = (t256 + 255) / 256 * 1000, cost192 = (t192 + 255) / 256 * 815,
-                    cost320 = (t320 + 255) / 256 * 1220;
+    const long long cost256 = rounds(t256) * 1000, cost192 = rounds(t192) * 815, cost320 = rounds(t320) * 1220;
     // Tiles of 256 rows x 128 tokens, 0.65 of the time of 256 x 256, where the last tile of 256 tokens
     // would be mostly empty (57,344 gated rows at K = 8192: 96 tokens 143 us against 224, 288 tokens 375
     // against 414).
     const long long t128t = (long long)((m + 127) / 128) * ((n + 255) / 256);
-    const long long cost128t = (t128t + 255) / 256 * 650;
+    const long long cost128t = rounds(t128t) * 650;
     // A very deep product in 2 K slices of the 256 x 256 tiles where that fills the last round better (8,192
     // rows at K = 28672, 3,072 tokens: 384 tiles, one and a half rounds that take the time of two; 768 half
     // tiles make three rounds of half the time: 1,125 us against 1,300, and 40 us for the second slab).
     if (epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 128) {
-      const long long cost256x2 = (2 * t256 + 255) / 256 * 500 + 60;
+      const long long cost256x2 = rounds(2 * t256) * 500 + 60;
       if (cost256x2 < cost256 && cost256x2 < cost192 && cost256x2 < cost320 && cost256x2 < cost128t) return {4, 2};
     }
     if (cost128t < cost256 && cost128t < cost192 && cost128t < cost320) return {8, 1};
@@ -695,22 +698,22 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   // A deep product (K >= 8192) whose 256 x 256 tiles are half a round goes in 2 slices of those
   // rather than in one round of the 256 x 128 tiles (4,096 rows at K = 14336: 2,048 tokens 197 us
   // against 220, 1,536 tokens 172 against 195; the second slab costs the norm that adds it about 10).
-  if (m > 64 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 64 && t256 * 2 >= 192 && t256 * 2 <= 256)
+  if (m > 64 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 64 && t256 * 2 >= R * 3 / 4 && t256 * 2 <= R)
     return {4, 2};
   // and where they are a quarter of a round, in 4 slices (768 tokens: 94 us against 106 in 2 slices of the
   // 256 x 128 tiles; 1,024 tokens: 109 against 118)
-  if (m > 64 && epilogue == 0 && (k / 64) % 4 == 0 && k / 64 / 4 >= 48 && t256 * 4 >= 192 && t256 * 4 <= 256)
+  if (m > 64 && epilogue == 0 && (k / 64) % 4 == 0 && k / 64 / 4 >= 48 && t256 * 4 >= R * 3 / 4 && t256 * 4 <= R)
     return {4, 4};
   // an eighth of a round, of a very deep product, in 8 (8,192 rows at K = 28672, 256 tokens: 122 us against 141
   // in 4 slices of the 256 x 128 tiles)
-  if (m > 128 && epilogue == 0 && (k / 64) % 8 == 0 && k / 64 / 8 >= 48 && t256 * 8 >= 192 && t256 * 8 <= 256)
+  if (m > 128 && epilogue == 0 && (k / 64) % 8 == 0 && k / 64 / 8 >= 48 && t256 * 8 >= R * 3 / 4 && t256 * 8 <= R)
     return {4, 8};
   // (a gated product, whose K cannot be cut, from 160 such tiles on: 22,016 gated rows, 256 tokens, 172
   // tiles 64 us against 74 in 344 tiles of 128 x 128)
-  if (m > 64 && t256x128 >= (epilogue == 1 ? 160 : 192) && t256x128 <= 256) return {8, 1};
+  if (m > 64 && t256x128 >= (epilogue == 1 ? R * 5 / 8 : R * 3 / 4) && t256x128 <= R) return {8, 1};
   if (m > 64 && epilogue == 0) {
     for (int p = 2; p <= 8; p *= 2)
-      if (t256x128 * p >= 160 && t256x128 * p <= 256 && (k / 64) % p == 0 && k / 64 / p >= (p == 2 ? 32 : (p == 4 ? (n <= 8192 ? 16 : 32) : 24)))
+      if (t256x128 * p >= R * 5 / 8 && t256x128 * p <= R && (k / 64) % p == 0 && k / 64 / p >= (p == 2 ? 32 : (p == 4 ? (n <= 8192 ? 16 : 32) : 24)))
         return {8, p};
   }
   // Between one and two thousand tokens the large tiles are too few for a round by themselves: a deep
@@ -719,16 +722,16 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   // 192 x 256 tiles alone make most of a round they are taken (1,408 tokens by 6,144 rows: 86 against 110).
   const long long t192r = (long long)((m + 255) / 256) * ((n + 191) / 192);
   if (m > 64 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 64) {
-    if (t192r * 2 >= 160 && t192r * 2 <= 256) return {6, 2};
-    if (t256 * 2 >= 160 && t256 * 2 <= 256) return {4, 2};
+    if (t192r * 2 >= R * 5 / 8 && t192r * 2 <= R) return {6, 2};
+    if (t256 * 2 >= R * 5 / 8 && t256 * 2 <= R) return {4, 2};
   }
   // (at K = 4096 where the 192-row tiles in 2 slices make three quarters of a round or more, up to 768
   // tokens, beyond which the second slab costs more than that: 12,288 rows, 384 tokens 51 us against 65;
   // 6,144 rows, 768 tokens 50 against 60)
-  if (m > 64 && m <= 768 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 32 && t192r * 2 >= 192 && t192r * 2 <= 256)
+  if (m > 64 && m <= 768 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 32 && t192r * 2 >= R * 3 / 4 && t192r * 2 <= R)
     return {6, 2};
-  if (m > 64 && t192r >= 176 && t192r <= 256) return {6, 1};
-  if (m > 64 && (t128 >= 256 || m > 512)) return {5, epilogue ? 1 : k_slices(t128, k, 512, k / (4 * m))};
+  if (m > 64 && t192r >= R * 11 / 16 && t192r <= R) return {6, 1};
+  if (m > 64 && (t128 >= R || m > 512)) return {5, epilogue ? 1 : k_slices(t128, k, 2 * R, k / (4 * m))};
   // A gated product of at most 64 tokens cannot cut K and streams W from too few workgroups to
   // hide anything (28,672 rows: 224 tiles of 128): tiles of 64 rows, four stages deep, two to a
   // compute unit, up to 24 tokens (17 tokens: 45 us against 50), and K tiles of 128 (256 bytes a
@@ -737,7 +740,7 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   // tiles, 17 tokens: 37 us against 34 with K tiles of 128), and with a deep K the plain 128 x 64 tiles
   // (57,344 gated rows at K = 8192: 139-147 us against 146-155 at 17 to 64 tokens).
   if (m <= 64 && epilogue == 1 && n >= 16384 && k < 8192) {
-    if (m <= 24 && (n + 63) / 64 >= 384) return {10, 1};
+    if (m <= 24 && (n + 63) / 64 >= R * 3 / 2) return {10, 1};
     if (k % 128 == 0) return {13, 1};
   }
   // At most 64 tokens, no gate: tiles of 128 rows in K slices, or tiles of 64 rows (four stages deep, two
@@ -749,13 +752,13 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
   // large tiles win at equal numbers (4,096 rows at K = 14336: 22.2 us against 23.3), and so they do
   // against small tiles in one slice (10,240 rows at K = 8192: 35.3 against 40.2).
   if (m <= 64 && epilogue == 0) {
-    const int pa = k_slices(t64, k, 256, k / (8 * m));
-    const int pb = k_slices((n + 63) / 64, k, 256, 8);
+    const int pa = k_slices(t64, k, R, k / (8 * m));
+    const int pb = k_slices((n + 63) / 64, k, R, 8);
     const long long wa = t64 * pa, wb = (long long)((n + 63) / 64) * pb;
-    if (wb <= 256 && (wb > wa || (wb == wa && pb >= 2 && k <= 8192))) return {10, pb};
+    if (wb <= R && (wb > wa || (wb == wa && pb >= 2 && k <= 8192))) return {10, pb};
     return {7, pa};
   }
-  return {7, epilogue ? 1 : k_slices(t64, k, 256, k / (8 * m))};
+  return {7, epilogue ? 1 : k_slices(t64, k, R, k / (8 * m))};
 }
 
 template <int EPI, typename TO, bool WF>
@@ -791,6 +794,12 @@ static int launch_planned(const bf16_t* x, const bf16_t* w, void* c, float* work
 #define RB_BY_OUTPUT(FN, WF, ...)                                                              \
   (epilogue == 0 ? (dtype_out == RB_F32 ? FN<0, float, WF>(__VA_ARGS__) : FN<0, bf16_t, WF>(__VA_ARGS__)) \
                  : (dtype_out == RB_F32 ? FN<1, float, WF>(__VA_ARGS__) : FN<1, bf16_t, WF>(__VA_ARGS__)))
+
+// what the planner picks for these sizes, as 100 * cfg + parts (0: not a product for this file)
+extern "C" int rb_tune_plan(int m, int n, int k, int epilogue) {
+  const TilePlan plan = plan_tiles(m, n, k, epilogue);
+  return plan.cfg == 0 ? 0 : 100 * plan.cfg + plan.parts;
+}
 
 int gemm_tiled_parts(int m, int n, int k, int epilogue) {
   const TilePlan plan = plan_tiles(m, n, k, epilogue);

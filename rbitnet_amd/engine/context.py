@@ -41,7 +41,7 @@ def bucket_max_pages(bucket: int) -> int:
     return None if bucket >= 16 else 16 * bucket - 1
 
 
-def decode_splits(n_seqs: int, n_kv_heads: int, bucket: int = 16, n_compute_units: int = 256) -> int:
+def decode_splits(n_seqs: int, n_kv_heads: int, bucket: int, n_compute_units: int) -> int:
     """Into how many workgroups the pages of one (sequence, kv head) are dealt in decode
     attention: what the context length asks for (`split_bucket`), but no more than gives
     every compute unit about one workgroup (every split adds to the combination)."""
@@ -89,7 +89,7 @@ def forget_step_array(name: str) -> None:
 
 class StepContext:
     def __init__(self, device, n_seqs: int, n_tokens: int, n_rows: int, table_widths: Dict[int, int],
-                 bucket: Optional[int] = None, n_compute_units: int = 256):
+                 bucket: Optional[int] = None, *, n_compute_units: int):
         """bucket: the split bucket of decode attention when it must not follow the batch (a
         captured step's grid cannot change); None: from each batch's longest context."""
         b, t = int(n_seqs), int(n_tokens)
@@ -142,7 +142,7 @@ class StepContext:
         self._workspaces: Dict[Tuple[int, int, int, int], Tuple] = {}
 
     @classmethod
-    def for_batch(cls, device, batch: StepBatch, n_compute_units: int = 256) -> "StepContext":
+    def for_batch(cls, device, batch: StepBatch, n_compute_units: int) -> "StepContext":
         widths = {key: max(1, max(len(r) for r in table)) for key, table in batch.block_tables.items()}
         ctx = cls(device, len(batch.slots), sum(len(t) for t in batch.tokens), len(batch.rows), widths,
                   n_compute_units=n_compute_units)

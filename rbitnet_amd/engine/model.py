@@ -1,11 +1,11 @@
-"""A model put together from a `ModelSpec`: embedding table, blocks, final norm, output
-matrix.  Nothing here knows an architecture: the spec says which parts and which tensor
-names, the part registries supply the parts.
+"""A model put together from a `ModelSpec`: an embedding, blocks, a head.  Nothing here knows
+an architecture, and the forward pass holds no stage of its own: the spec says which parts and
+which tensor names, the part registries supply the parts.
 
 The forward pass of one step follows the reference's per-token order
 (crates/bitnet-core/src/llama/model.rs:229-315): embedding row, the layers in schedule
-order, final norm and output matrix -- the last two only on the rows whose logits were
-asked for.
+order, final norm and output matrix -- the last two (the head) only on the rows whose logits
+were asked for.
 """
 from __future__ import annotations
 
@@ -16,8 +16,7 @@ import torch
 from ..config.spec import ModelSpec
 from ..errors import ConfigError
 from ..parts.base import BuildEnv, CacheRequest, TensorSpec, build_part
-from ..parts.block import normed_for
-from ..parts.linear import linear, pack_rows
+from ..parts.stream import run_blocks
 
 
 def _build_blocks(spec: ModelSpec, env_for: Callable[[int], BuildEnv]):
@@ -31,8 +30,12 @@ def _build_blocks(spec: ModelSpec, env_for: Callable[[int], BuildEnv]):
     return blocks
 
 
-def _named_parts(spec: ModelSpec, blocks, final_norm) -> Dict[str, object]:
-    """prefix -> part, for every part that owns tensors."""
+def _ends(spec: ModelSpec, env: BuildEnv):
+    return build_part("embedding", spec.embedding, env), build_part("head", spec.head, env)
+
+
+def _named_parts(spec: ModelSpec, blocks) -> Dict[str, object]:
+    """prefix -> part, for every part of a block that owns tensors (the two ends name theirs in full)."""
     out: Dict[str, object] = {}
     for layer, block in zip(spec.layers, blocks):
         for segment, part in block.parts().items():
@@ -40,32 +43,25 @@ def _named_parts(spec: ModelSpec, blocks, final_norm) -> Dict[str, object]:
     return out
 
 
+def _expected(spec: ModelSpec, blocks, embedding, head) -> Dict[str, TensorSpec]:
+    out: Dict[str, TensorSpec] = {}
+    for part in (embedding, head):
+        out.update(part.tensor_specs())
+    for prefix, part in _named_parts(spec, blocks).items():
+        for name, ts in part.tensor_specs().items():
+            out[f"{prefix}.{name}"] = ts
+    return out
+
+
 def expected_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:
     """Every tensor the model's parts declare, by full name, without touching a GPU."""
     env = BuildEnv(hidden_size=spec.hidden_size, dtype=torch.float32, device=torch.device("cpu"), lib=None)
     blocks = _build_blocks(spec, lambda i: env)
-    final_norm = build_part("norm", spec.final_norm, env)
-    out: Dict[str, TensorSpec] = {
-        spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden_size)),
-    }
-    for prefix, part in _named_parts(spec, blocks, final_norm).items():
-        for name, ts in part.tensor_specs().items():
-            out[f"{prefix}.{name}"] = ts
-    norm_specs = final_norm.tensor_specs()
-    if len(norm_specs) == 1:
-        out[spec.final_norm_name] = next(iter(norm_specs.values()))
-    else:
-        base = spec.final_norm_name.rsplit(".", 1)[0]
-        for name, ts in norm_specs.items():
-            out[f"{base}.{name}"] = ts
-    if spec.head_name is not None:
-        out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size))
-    return out
+    embedding, head = _ends(spec, env)
+    return _expected(spec, blocks, embedding, head)
 
 
 class Model:
-    takes_gained_rows = True      # the output product takes what the last product left for the final norm
-
     def __init__(self, spec: ModelSpec, dtype: torch.dtype, device, lib, generic_only: bool = False,
                  max_seq_len: Optional[int] = None):
         if dtype not in (torch.float32, torch.bfloat16):
@@ -86,10 +82,8 @@ class Model:
             return env
 
         self.blocks = _build_blocks(spec, env_for)
-        self.final_norm = build_part("norm", spec.final_norm, env_for(-1))
-        self.embedding: Optional[torch.Tensor] = None
-        self.head: Optional[torch.Tensor] = None
-        self.expected = expected_tensors(spec)
+        self.embedding, self.head = _ends(spec, env_for(-1))
+        self.expected = _expected(spec, self.blocks, self.embedding, self.head)
 
     # ------------------------------------------------------------------ cache needs
     def cache_requests(self) -> List[Optional[CacheRequest]]:
@@ -123,8 +117,7 @@ class Model:
 
     @property
     def graph_safe(self) -> bool:
-        return (all(getattr(b, "graph_safe", False) for b in self.blocks)
-                and getattr(self.final_norm, "graph_safe", False))
+        return all(getattr(p, "graph_safe", False) for p in list(self.blocks) + [self.embedding, self.head])
 
     def max_positions(self) -> int:
         return self.spec.max_positions
@@ -150,54 +143,38 @@ class Model:
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         """tensors: full name -> tensor (any device, stored dtype).  Each is moved to the
         GPU in the dtype its role asks for and handed to its part."""
-        spec = self.spec
         placed = lambda name: self._place(tensors[name], self.expected[name])
-        self.embedding = placed(spec.embedding_name)
-        if spec.head_name is None:
-            self.head = self.embedding            # tied: the table's rows are also read one by one
-        else:
-            head = placed(spec.head_name)
-            self.head = pack_rows(self.lib, [(head, 0, None, None)], head.shape[0], head.shape[1], head.dtype,
-                                  head.device, not self.generic_only)
-        for prefix, part in _named_parts(spec, self.blocks, self.final_norm).items():
+        self.embedding.load({name: placed(name) for name in self.embedding.tensor_specs()})
+        self.head.load({name: placed(name) for name in self.head.tensor_specs()}, embedding=self.embedding)
+        for prefix, part in _named_parts(self.spec, self.blocks).items():
             part.load({name: placed(f"{prefix}.{name}") for name in part.tensor_specs()})
-        norm_specs = self.final_norm.tensor_specs()
-        if len(norm_specs) == 1:
-            self.final_norm.load({next(iter(norm_specs)): placed(spec.final_norm_name)})
-        else:
-            base = spec.final_norm_name.rsplit(".", 1)[0]
-            self.final_norm.load({name: placed(f"{base}.{name}") for name in norm_specs})
 
     def weight_bytes(self) -> int:
-        """Bytes of every weight a step reads once (a tied head counts once more: it is
-        read again as the output matrix)."""
+        """Bytes of every weight a step reads once: all tensors of the blocks, and of the two ends
+        what they say (`step_bytes`: a table that is only gathered from counts nothing, a matrix
+        shared with it counts where it is read in full)."""
+        esize = 4 if self.dtype == torch.float32 else 2
         total = 0
-        for name, ts in self.expected.items():
-            n = 1
-            for s in ts.shape:
-                n *= s
-            if name == self.spec.embedding_name:
-                continue          # the gather reads a few rows only
-            total += n * (4 if ts.role in ("gain", "table") or self.dtype == torch.float32 else 2)
-        if self.spec.head_name is None:
-            total += self.spec.vocab_size * self.spec.hidden_size * (4 if self.dtype == torch.float32 else 2)
+        for prefix, part in _named_parts(self.spec, self.blocks).items():
+            total += _tensor_bytes(part.tensor_specs().values(), esize)
+        for part in (self.embedding, self.head):
+            own = getattr(part, "step_bytes", None)
+            total += own(esize) if own else _tensor_bytes(part.tensor_specs().values(), esize)
         return total
 
     # ------------------------------------------------------------------ forward
     def forward(self, ctx, cache, rows: torch.Tensor) -> torch.Tensor:
         """ctx.token_ids [T] -> float32 logits [len(rows), V] at the packed rows `rows`."""
-        x = torch.empty((ctx.n_tokens, self.spec.hidden_size), dtype=torch.float32, device=self.device)
-        self.lib.embed_gather(self.embedding, ctx.token_ids, x)
-        pending = None
-        schedule = self.spec.schedule
-        for place, i in enumerate(schedule):
-            block = self.blocks[i]
-            view = cache.view(place, ctx.block_tables)
-            if getattr(block, "takes_next_norm", False):
-                after = self.blocks[schedule[place + 1]] if place + 1 < len(schedule) else None
-                next_norm = self.final_norm if after is None else getattr(after, "first_norm", None)
-                pending = block.forward(x, pending, ctx, view, next_norm=next_norm)
-            else:
-                pending = block.forward(x, pending, ctx, view)
-        xn = normed_for(self, self.final_norm, x, pending, rows)
-        return linear(self.lib, xn, self.head, torch.float32)
+        x = self.embedding.forward(ctx)
+        pending = run_blocks(self.blocks, self.spec.schedule, x, ctx, cache, getattr(self.head, "first_norm", None))
+        return self.head.forward(x, pending, rows, ctx)
+
+
+def _tensor_bytes(specs, element_size: int) -> int:
+    total = 0
+    for ts in specs:
+        n = 1
+        for s in ts.shape:
+            n *= s
+        total += n * (4 if ts.role in ("gain", "table") else element_size)
+    return total

@@ -7,6 +7,8 @@ Kinds of parts and the registry each lives in:
 * mixer           `register_mixer`          forward(h [T, E], ctx, view) -> [T, E_out]
 * feed-forward    `register_feed_forward`   forward(h [T, E], ctx) -> [T, E]
 * block           `register_block`          arranges norm, mixer, norm, feed-forward
+* embedding       `register_embedding`      forward(ctx) -> x [T, E], the residual stream
+* head            `register_head`           forward(x, pending, rows, ctx) -> logits [rows, V]
 
 A part is built from `(params, env)`: `params` is the dict of its `PartSpec`,
 `env` a `BuildEnv` (model width, compute dtype, device, the kernel library).
@@ -90,7 +92,7 @@ class Part:
 
 
 _REGISTRIES: Dict[str, Dict[str, Callable[..., Any]]] = {
-    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {},
+    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {}, "head": {},
 }
 
 
@@ -116,6 +118,14 @@ def register_feed_forward(kind: str, factory: Callable[..., Any]) -> None:
 
 def register_block(kind: str, factory: Callable[..., Any]) -> None:
     _register("block", kind, factory)
+
+
+def register_embedding(kind: str, factory: Callable[..., Any]) -> None:
+    _register("embedding", kind, factory)
+
+
+def register_head(kind: str, factory: Callable[..., Any]) -> None:
+    _register("head", kind, factory)
 
 
 def build_part(group: str, spec: Any, env: BuildEnv) -> Any:

@@ -6,10 +6,9 @@ The residual stream x is float32 and each sum is done by the norm that follows i
 norm.py), so a block takes the previous block's not yet added output as `pending` and
 returns its own.  The model adds the last one in the final norm.
 
-A part that says `adds_to_stream` is given the stream and the norm that follows and may add
-its output itself; it then returns None, or the rows as its last product prepared them for
-that norm (`GainedRows`), which go to the next part if it says `takes_gained_rows`.  With
-both, a step of a few tokens runs no kernel between the products.
+Who adds what to the stream, and in which form a part's output travels to the next norm, is
+`stream.py`'s business: an arrangement calls `sublayer(part, norm, x, pending, next_norm, ...)`
+once per part and hands on what comes back.
 
 Interface of a block: parts() -> {name: part} for the loader (names are tensor-name
 segments below the layer's prefix); mixer (for the cache request);
@@ -19,12 +18,12 @@ forward then also takes next_norm, the first norm of whatever runs after it.
 """
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Dict
 
 import torch
 
 from .base import BuildEnv, build_part, register_block
-from .norm import GainedRows
+from .stream import normed_for, sublayer  # noqa: F401  (normed_for: its old home)
 
 DEFAULT_SEGMENTS = {"norm1": "input_layernorm", "mixer": "self_attn", "norm2": "post_attention_layernorm",
                     "feed_forward": "mlp"}
@@ -53,26 +52,8 @@ class PreNormBlock:
         return self.norm1
 
     def forward(self, x: torch.Tensor, pending, ctx, view, next_norm=None):
-        h = normed_for(self.mixer, self.norm1, x, pending)
-        if getattr(self.mixer, "adds_to_stream", False):
-            a = self.mixer.forward(h, ctx, view, stream=x, next_norm=self.norm2)
-        else:
-            a = self.mixer.forward(h, ctx, view)
-        h2 = normed_for(self.feed_forward, self.norm2, x, a)
-        if getattr(self.feed_forward, "adds_to_stream", False):
-            return self.feed_forward.forward(h2, ctx, stream=x, next_norm=next_norm)
-        return self.feed_forward.forward(h2, ctx)
-
-
-def normed_for(part, norm, x: torch.Tensor, pending, rows: Optional[torch.Tensor] = None):
-    """The input of `part`: the stream x, with `pending` added if that is a tensor, normalised
-    by `norm` (all rows, or `rows`).  GainedRows that were made for this norm go on as they are
-    to a part that takes them."""
-    if isinstance(pending, GainedRows):
-        if pending.norm is norm and getattr(part, "takes_gained_rows", False):
-            return pending.select(rows)
-        return norm.forward(x, None, rows)         # the stream holds the sum already
-    return norm.forward(x, pending, rows)
+        a = sublayer(self.mixer, self.norm1, x, pending, self.norm2, ctx, view)
+        return sublayer(self.feed_forward, self.norm2, x, a, next_norm, ctx)
 
 
 register_block("prenorm", PreNormBlock)

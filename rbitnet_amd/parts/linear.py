@@ -17,7 +17,7 @@ from typing import Optional
 import torch
 
 from ..errors import KernelError
-from .norm import GainedRows
+from .stream import GainedRows, norm_adds_terms, norm_folds
 
 GATE_BLOCK = 16     # rows per block when gate and up rows are interleaved for the fused epilogue
 
@@ -114,11 +114,11 @@ def linear_to_stream(lib, x: torch.Tensor, w, stream: Optional[torch.Tensor], ne
     wd, frag = _data(w)
     if stream is None or x.shape[0] == 0 or not _few(lib, x, w):
         m, k = x.shape
-        if (next_norm is not None and getattr(next_norm, "adds_terms", False) and uses_matrix_cores(x.dtype, k)
+        if (norm_adds_terms(next_norm) and uses_matrix_cores(x.dtype, k)
                 and lib.gemm_bf16_terms_count(m, w.shape[0], k) > 1):
             return lib.gemm_bf16_terms(x, wd, w_frag=frag)        # [P, M, N]: the norm adds them up with the stream
         return linear(lib, x, w, torch.float32)
-    if next_norm is None or not getattr(next_norm, "folds_into_products", False):
+    if not norm_folds(next_norm):
         lib.gemm_bf16_few(x, wd, stream, 2, w_frag=frag)
         return None
     m, n = stream.shape

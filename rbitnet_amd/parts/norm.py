@@ -24,36 +24,7 @@ from typing import Dict, Optional
 import torch
 
 from .base import BuildEnv, Part, TensorSpec, register_norm
-
-
-class GainedRows:
-    """Rows of the float32 stream `x` (all, or those `rows` names) as a product left them for
-    `norm`: gained [T, E] = bf16(x * gain) and squares [T, ceil(E / 16)], the sums of x^2 over
-    every 16 columns.  What is left of the norm is one factor per row.  `linear` takes them as
-    tokens; tensor() normalises the rows with the norm's own kernel instead.  shape, dtype and
-    device are those of the normalised rows."""
-
-    def __init__(self, norm: "RMSNorm", x: torch.Tensor, gained: torch.Tensor, squares: torch.Tensor,
-                 rows: Optional[torch.Tensor] = None):
-        self.norm = norm
-        self.x = x
-        self.gained = gained
-        self.squares = squares
-        self.rows = rows
-        self.eps = norm.eps
-        self.shape = (x.shape[0] if rows is None else rows.shape[0], norm.size)
-        self.dtype = norm.env.dtype
-        self.device = x.device
-
-    def select(self, rows: Optional[torch.Tensor]) -> "GainedRows":
-        if rows is None:
-            return self
-        if self.rows is not None:
-            raise ValueError("rows were chosen already")
-        return GainedRows(self.norm, self.x, self.gained, self.squares, rows)
-
-    def tensor(self) -> torch.Tensor:
-        return self.norm.forward(self.x, None, self.rows)
+from .stream import GainedRows  # noqa: F401  (its old home; importers find it here too)
 
 
 class RMSNorm(Part):

@@ -97,8 +97,8 @@ def test_prompts_in_pieces_for_several_sequences_at_once(name, dtype):
     """Steps that bring several tokens per sequence on top of pasts that differ per sequence (a
     prompt fed in pieces, batched): pieces that end inside a page, at its edge and beyond it, a
     sequence that brings one token while its neighbours bring many."""
-    lengths = [130, 64, 75]
-    cuts = [[60, 5, 64], [4, 59, 1], [66, 0, 9]]            # tokens per sequence and step; 0: it sits the step out
+    lengths = [125, 64, 75]
+    cuts = [[60, 5, 64], [4, 59, 1], [61, 0, 10]]           # tokens per sequence and step; 0: it sits the step out
     reqs = [tokens_for(name, n, 60 + i) for i, n in enumerate(lengths)]
     eng = _engine(name, dtype, max_batch=3, max_tokens=64 * 5)
     for g in eng.cache.kv_groups:

@@ -176,11 +176,11 @@ def test_decode_attention_split_rule(monkeypatch):
     for b in (1, 2, 4, 8):
         assert split_bucket(64 * bucket_max_pages(b)) == b and split_bucket(64 * bucket_max_pages(b) + 1) == 2 * b
     assert bucket_max_pages(16) is None
-    assert decode_splits(8, 8, split_bucket(600)) == 1
-    assert decode_splits(8, 8, split_bucket(4096)) == 4          # 256 // (8 * 8)
-    assert decode_splits(1, 8, split_bucket(4096)) == 8
-    assert decode_splits(64, 8, split_bucket(65536)) == 1
-    assert decode_splits(1, 1, 16) == 16
+    assert decode_splits(8, 8, split_bucket(600), 256) == 1
+    assert decode_splits(8, 8, split_bucket(4096), 256) == 4     # 256 // (8 * 8)
+    assert decode_splits(1, 8, split_bucket(4096), 256) == 8
+    assert decode_splits(64, 8, split_bucket(65536), 256) == 1
+    assert decode_splits(1, 1, 16, 256) == 16
     assert decode_splits(8, 8, 16, n_compute_units=128) == 2     # a smaller GPU
     monkeypatch.setattr(context, "FORCED_DECODE_SPLITS", 3)
-    assert decode_splits(64, 8, 1) == 3
+    assert decode_splits(64, 8, 1, 256) == 3

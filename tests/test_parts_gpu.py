@@ -42,9 +42,11 @@ def _ctx_and_cache(part, past, tokens_per_seq, dtype):
 
 
 def _step(cache, slots, q_lens):
+    from rbitnet_amd.csrc.lib import kernels
     past = [cache.length(s) for s in slots]
     cache.reserve(slots, q_lens)
-    return StepContext.for_batch(DEV, StepBatch(slots, past, [[0] * q for q in q_lens], [], cache.block_tables(slots)))
+    return StepContext.for_batch(DEV, StepBatch(slots, past, [[0] * q for q in q_lens], [], cache.block_tables(slots)),
+                                 n_compute_units=kernels().n_compute_units)
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-6), (torch.bfloat16, 8e-3)])
@@ -515,3 +517,117 @@ def test_toy_position_and_routed_feed_forward():
             assert _rel(logits[i:i + 1], w[c + j:c + j + 1]) < 4e-2
     for sl in slots:
         eng.free_slot(sl)
+
+
+class ScaledTable(Part):
+    """An embedding of the test's own: the row of the table times a constant (as architectures
+    that multiply their embeddings by sqrt(width) do)."""
+    graph_safe = True
+
+    def __init__(self, params, env):
+        self.env, self.name, self.vocab, self.scale = env, params["name"], int(params["vocab_size"]), float(params["scale"])
+
+    def tensor_specs(self):
+        return {self.name: TensorSpec((self.vocab, self.env.hidden_size))}
+
+    def load(self, tensors):
+        self.table = tensors[self.name]
+
+    def step_bytes(self, element_size):
+        return 0
+
+    def forward(self, ctx):
+        return self.table.float().index_select(0, ctx.token_ids.long()) * self.scale
+
+
+class CappedHead(Part):
+    """A head of the test's own: no sharing with the embedding, a norm of its own kind and name,
+    and logits squeezed into (-cap, cap): cap * tanh(W norm(x) / cap)."""
+    graph_safe = True
+
+    def __init__(self, params, env):
+        self.env, self.cap, self.vocab = env, float(params["cap"]), int(params["vocab_size"])
+        self.norm = build_part("norm", params["norm"], env)
+
+    @property
+    def first_norm(self):
+        return self.norm
+
+    def tensor_specs(self):
+        return {"out.norm.weight": self.norm.tensor_specs()["weight"],
+                "out.proj.weight": TensorSpec((self.vocab, self.env.hidden_size))}
+
+    def load(self, tensors, embedding=None):
+        self.norm.load({"weight": tensors["out.norm.weight"]})
+        self.w = tensors["out.proj.weight"]
+
+    def forward(self, x, pending, rows, ctx=None):
+        from rbitnet_amd.parts.linear import linear
+        from rbitnet_amd.parts.stream import normed_for
+        z = linear(self.env.lib, normed_for(None, self.norm, x, pending, rows), self.w, torch.float32)
+        return self.cap * torch.tanh(z / self.cap)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_embedding_with_a_scale_and_capped_head_registered_from_here(dtype, tol):
+    """The two ends of a model are parts like the others: another embedding and another head are
+    registered here, named in a hand-made spec and run by the engine's step and its captured
+    decode step, with no change to the package."""
+    import rbitnet_amd
+    from rbitnet_amd.engine.model import expected_tensors
+    from rbitnet_amd.parts import register_embedding, register_head
+    from rbitnet_amd.weights import random_tensors
+    register_embedding("scaled_table", ScaledTable)
+    register_head("capped", CappedHead)
+    hidden, vocab, scale, cap = 64, 75, 3.5, 2.0
+    norm = PartSpec("rmsnorm", {"size": hidden, "eps": 1e-5})
+    att = _attention_params(4, 2, 16, window=None)
+    layers = [LayerSpec(f"blocks.{i}", "prenorm", PartSpec("attention", att), PartSpec("swiglu", {"intermediate_size": 48}),
+                        norm, norm) for i in range(2)]
+    spec = ModelSpec(architecture="ToyForTests", hidden_size=hidden, vocab_size=vocab, max_positions=256, layers=layers,
+                     embedding=PartSpec("scaled_table", {"name": "tokens.weight", "vocab_size": vocab, "scale": scale}),
+                     head=PartSpec("capped", {"norm": norm, "vocab_size": vocab, "cap": cap}))
+    expected = expected_tensors(spec)
+    assert {"tokens.weight", "out.norm.weight", "out.proj.weight"} <= set(expected)
+    tensors = dict(random_tensors(expected, seed=9, std=0.15, norm_std=0.05, dtype=torch.bfloat16))
+    tensors["out.proj.weight"] = tensors["out.proj.weight"] * 6          # logits large enough for the cap to bend them
+
+    def plain(tokens):
+        # the plain Llama layers between the test's own ends
+        w = {k: v.double().cpu() for k, v in tensors.items()}
+        x = P.embedding(w["tokens.weight"], tokens) * scale
+        for i in range(2):
+            pre = f"blocks.{i}"
+            h = P.rmsnorm(x, w[f"{pre}.input_layernorm.weight"], 1e-5)
+            inv = P.rope_inv_freq(16, att["position"]["theta"], None)
+            q, k, v = (P.linear(h, w[f"{pre}.self_attn.{n}_proj.weight"]) for n in "qkv")
+            q, k = P.rope_rows(q, 4, inv), P.rope_rows(k, 2, inv)
+            x = x + P.linear(P.attention(q, k, v, 4, 2), w[f"{pre}.self_attn.o_proj.weight"])
+            h2 = P.rmsnorm(x, w[f"{pre}.post_attention_layernorm.weight"], 1e-5)
+            x = x + P.swiglu(h2, w[f"{pre}.mlp.gate_proj.weight"], w[f"{pre}.mlp.up_proj.weight"],
+                             w[f"{pre}.mlp.down_proj.weight"])
+        z = P.linear(P.rmsnorm(x, w["out.norm.weight"], 1e-5), w["out.proj.weight"])
+        return cap * torch.tanh(z / cap)
+
+    eng = rbitnet_amd.Engine.from_spec(spec, tensors, dtype=dtype, max_tokens=64 * 4, max_batch=2)
+    assert eng.use_graphs
+    g = torch.Generator().manual_seed(12)
+    seqs = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in (70, 12)]
+    want = [plain(s) for s in seqs]
+    assert float(want[0].abs().max()) > 0.9 * cap                         # the cap does bend them
+    slots = [eng.alloc_slot() for _ in seqs]
+    cut = [len(s) - 4 for s in seqs]
+    logits = eng.step([(sl, s[:c]) for sl, s, c in zip(slots, seqs, cut)], "all")
+    off = 0
+    for c, w in zip(cut, want):
+        assert _rel(logits[off:off + c], w[:c]) < tol
+        off += c
+    for j in range(4):                                                    # the captured decode step
+        eng.decode_step(slots, [s[c + j] for s, c in zip(seqs, cut)])
+        for i, (c, w) in enumerate(zip(cut, want)):
+            assert _rel(eng.last_decode_logits[i:i + 1], w[c + j:c + j + 1]) < tol
+    assert len(eng._graphs) == 1
+    # what a step reads: every tensor of the blocks, the head's two, nothing of the table
+    esize = 4 if dtype == "float32" else 2
+    per_layer = (64 * 64 * 2 + 2 * 32 * 64 + 3 * 48 * 64) * esize + 2 * 64 * 4
+    assert eng.model.weight_bytes() == 2 * per_layer + vocab * hidden * esize + hidden * 4
