@@ -109,6 +109,54 @@ def decode_run(engine, batch: int, steps: int, warmup: int, seed: int = 0, promp
     return dt, ctx_mean
 
 
+def generate_run(engine, n_requests: int, prompt_len: int, seed: int = 0, lo: int = 16, hi: int = 256) -> dict:
+    """`Engine.generate` for n requests whose limits are drawn from lo..hi, so that the batch
+    shrinks by a sequence every few steps: the loop's wall time for the decoding part (the prompts'
+    step is timed by itself and taken off) against the sum of what its steps take as captured
+    steps of a fixed batch of the same size, measured one size after the other."""
+    import numpy as np
+    from .engine.decode_graph import graph_size
+    rng = np.random.default_rng(seed)
+    vocab = engine.spec.vocab_size
+    prompts = [[int(t) for t in rng.integers(0, vocab, size=prompt_len)] for _ in range(n_requests)]
+    limits = [int(v) for v in rng.integers(lo, hi + 1, size=n_requests)]
+    # the prompts' step alone (twice: the first run warms up)
+    for _ in range(2):
+        slots = [engine.alloc_slot() for _ in prompts]
+        _sync()
+        t0 = time.perf_counter()
+        engine.step(list(zip(slots, prompts)), "last")
+        _sync()
+        t_prompt = time.perf_counter() - t0
+        for s in slots:
+            engine.free_slot(s)
+    walls = []
+    for _ in range(2):                      # the second run finds every size captured
+        _sync()
+        t0 = time.perf_counter()
+        results = engine.generate(prompts, max_tokens=limits, temperature=0.0, stop_token_ids=[])
+        _sync()
+        walls.append(time.perf_counter() - t0)
+    assert [len(r.tokens) for r in results] == limits
+    # a step feeds the sequences that have not yet reached their limit: step j (from 1) runs those with limit > j
+    sizes = [sum(1 for m in limits if m > j) for j in range(1, max(limits))]
+    per_size = {}
+    for b in sorted(set(graph_size(v) for v in sizes if v)):
+        dt, _ = decode_run(engine, b, 24, 4, seed=100 + b, prompt_len=prompt_len)
+        per_size[b] = dt / 24
+    expected = sum(per_size[graph_size(v)] for v in sizes if v)
+    decoded = sum(limits) - n_requests          # every request's first token comes from the prompts' step
+    out = {"requests": n_requests, "prompt_len": prompt_len, "new_tokens": sum(limits), "steps": len(sizes),
+           "prompt_step_ms": round(t_prompt * 1e3, 2)}
+    for label, wall in (("first_run", walls[0]), ("second_run", walls[1])):
+        loop = wall - t_prompt
+        out[label] = {"wall_ms": round(wall * 1e3, 1), "decode_ms": round(loop * 1e3, 1),
+                      "decode_tokens_per_s": round(decoded / loop, 1), "over_fixed_batches": round(loop / expected, 3)}
+    out["fixed_batches_ms"] = round(expected * 1e3, 1)
+    out["fixed_batch_tokens_per_s"] = {str(b): round(b / t, 1) for b, t in per_size.items()}
+    return out
+
+
 def probe(lib, device) -> dict:
     """What this GPU reaches on a streaming read (`read_*`: all workgroups striding through the
     buffer together with plain loads; `stream_*`: every workgroup walking pieces of its own with
@@ -165,7 +213,11 @@ def main(argv=None) -> int:
     ap.add_argument("--planner-sweep", action="store_true",
                     help="no benchmark: time every product of the named shapes with the planner's choice and with "
                          "every choice forced (see planner_check.py)")
+    ap.add_argument("--generate", type=int, default=0, metavar="N",
+                    help="no benchmark line: Engine.generate for N requests with limits drawn from 16..256 against "
+                         "captured steps of fixed batches (see generate_run)")
     ap.add_argument("--tokens", default="1,8,64,512,2048", help="token counts of --planner-sweep")
+    ap.add_argument("--sweep-detail", default=None, help="--planner-sweep: a file for every candidate's time")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="length of the one prompt whose prefill is timed")
     ap.add_argument("--prompt-len", default=str(PROMPT_LEN),
@@ -181,7 +233,9 @@ def main(argv=None) -> int:
             ap.error(f"unknown --model {name!r}; one of {', '.join(sorted(MODELS))}")
     if args.planner_sweep:
         from .planner_check import sweep
-        sweep([(MODELS[n][0], MODELS[n][1]) for n in names], [int(v) for v in args.tokens.split(",") if v])
+        detail = open(args.sweep_detail, "w") if args.sweep_detail else None
+        sweep([(MODELS[n][0], MODELS[n][1]) for n in names], [int(v) for v in args.tokens.split(",") if v],
+              detail=detail)
         return 0
     if len(names) != 1:
         ap.error("one --model at a time")
@@ -201,7 +255,7 @@ def main(argv=None) -> int:
         cfg["num_hidden_layers"] = args.layers
     layers = cfg["num_hidden_layers"]
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
-    max_batch = max([args.batch] + ([] if args.no_points else [int(v) for v in args.points.split(",") if v]))
+    max_batch = max([args.batch, args.generate] + ([] if args.no_points else [int(v) for v in args.points.split(",") if v]))
     ctx_cap = longest + max(NEW_TOKENS, args.steps + args.warmup) + 64
     prefill_tokens = args.prefill_tokens
     max_tokens = max(max_batch * ctx_cap, prefill_tokens + 64)
@@ -211,6 +265,9 @@ def main(argv=None) -> int:
     engine = Engine.random(cfg, seed=0, dtype=dtype, std=0.02, norm_std=0.0, max_batch=max_batch,
                            max_tokens=max_tokens, max_seq_len=max_seq_len)
     _sync()
+    if args.generate:
+        print(json.dumps(generate_run(engine, args.generate, longest)))
+        return 0
 
     dt, ctx_mean = decode_run(engine, args.batch, args.steps, args.warmup, prompt_len=prompt_len)
     ms = dt / args.steps * 1e3

@@ -13,6 +13,29 @@
 * Nothing is cleared when a slot or a page is reused: only positions below a
   sequence's length are ever read (the reference zero-fills, model.rs:44-51, without
   needing to: it reads 0..=pos only, :266,279).
+* One page and one slot more than are ever handed out, the spare ones: a captured decode
+  step made for more sequences than are running fills its idle rows with a sequence of
+  length 0 in the spare slot, whose keys, values and state go to the spare page and the
+  spare state and nowhere else.
+
+A storage group is a class registered under the kind of a `CacheRequest`
+(`register_cache_kind`), built as `cls(request, layers, n_pages, n_slots, dtype, device)`:
+
+    kind                  the request kind it serves
+    open(slot), close(slot)
+    fill_view(view, i, block_tables)     what layer i of the group shows a mixer in a step
+    bytes()                              its storage
+    bytes_per_token(request, n_layers, dtype)      static: growth per token of a sequence
+
+and, when it grows with its sequences in pages (`paged = True`; derive from `PagedGroup`):
+
+    table                 a `PageTable` (ensure, release_behind, pages, pool)
+    pages_missing(slot, n_tokens)
+    spare_page            index of the page that idle rows write to (its storage holds
+                          n_pages + 1 pages)
+
+A group that keeps something per slot gives it room for n_slots + 1 slots.  Only a "kv"
+group can be read by another layer (`readers`): what is shared are keys and values.
 """
 from __future__ import annotations
 
@@ -35,22 +58,17 @@ class LayerCacheView:
     state: Optional[torch.Tensor] = None          # [slots, *shape]; index with ctx.slots
 
 
-class KvGroup:
-    """Keys and values per token in pages; a window gives pages back as a sequence moves on."""
-    kind = "kv"
+class PagedGroup:
+    """What the cache needs of a group that grows with its sequences in pages: a page table
+    over n_pages pages, and one page more that is never handed out."""
+    paged = True
 
-    def __init__(self, request: CacheRequest, layers: List[int], n_pages: int, n_slots: int, dtype, device):
+    def __init__(self, request: CacheRequest, layers: List[int], n_pages: int):
         self.request = request
         self.layers = list(layers)
         self.index = {l: i for i, l in enumerate(self.layers)}
         self.table = PageTable(n_pages, request.window)
-        shape = (len(self.layers), n_pages, request.heads, PAGE_SIZE, request.head_dim)
-        self.k = torch.empty(shape, dtype=dtype, device=device)
-        self.v = torch.empty(shape, dtype=dtype, device=device)
-
-    @staticmethod
-    def bytes_per_token(request: CacheRequest, n_layers: int, dtype: torch.dtype) -> int:
-        return 2 * n_layers * request.heads * request.head_dim * torch.empty((), dtype=dtype).element_size()
+        self.spare_page = int(n_pages)
 
     def open(self, slot: int) -> None:
         self.table.open(slot)
@@ -60,6 +78,21 @@ class KvGroup:
 
     def pages_missing(self, slot: int, n_tokens: int) -> int:
         return max(0, pages_for(n_tokens) - len(self.table.pages(slot)))
+
+
+class KvGroup(PagedGroup):
+    """Keys and values per token in pages; a window gives pages back as a sequence moves on."""
+    kind = "kv"
+
+    def __init__(self, request: CacheRequest, layers: List[int], n_pages: int, n_slots: int, dtype, device):
+        super().__init__(request, layers, n_pages)
+        shape = (len(self.layers), n_pages + 1, request.heads, PAGE_SIZE, request.head_dim)
+        self.k = torch.empty(shape, dtype=dtype, device=device)
+        self.v = torch.empty(shape, dtype=dtype, device=device)
+
+    @staticmethod
+    def bytes_per_token(request: CacheRequest, n_layers: int, dtype: torch.dtype) -> int:
+        return 2 * n_layers * request.heads * request.head_dim * torch.empty((), dtype=dtype).element_size()
 
     def fill_view(self, view: "LayerCacheView", i: int, block_tables: Dict[int, torch.Tensor]) -> None:
         view.k_pages, view.v_pages = self.k[i], self.v[i]
@@ -77,7 +110,7 @@ class StateGroup:
         self.request = request
         self.layers = list(layers)
         self.index = {l: i for i, l in enumerate(self.layers)}
-        shape = (len(self.layers), n_slots) + tuple(request.state_shape)
+        shape = (len(self.layers), n_slots + 1) + tuple(request.state_shape)        # the last: the spare slot's
         self.data = torch.full(shape, request.state_init, dtype=request.state_dtype, device=device)
 
     @staticmethod
@@ -97,11 +130,7 @@ class StateGroup:
         return self.data.numel() * self.data.element_size()
 
 
-# kind of a CacheRequest -> the class that stores it.  A group class has: kind,
-# __init__(request, layers, n_pages, n_slots, dtype, device), open(slot), close(slot),
-# fill_view(view, index in the group, block tables of the step), bytes() and the static
-# bytes_per_token(request, n_layers, dtype); one that grows with the sequence in pages keeps a
-# PageTable as `table`, as KvGroup does, and is then counted when pages are reserved.
+# kind of a CacheRequest -> the class that stores it (the interface: see the module's text)
 _GROUP_KINDS: Dict[str, type] = {"kv": KvGroup, "state": StateGroup}
 
 
@@ -130,6 +159,7 @@ class Cache:
         if n_slots <= 0:
             raise CacheError("the cache needs at least one slot")
         self.n_slots = int(n_slots)
+        self.spare_slot = self.n_slots          # never handed out: where idle rows of a captured step live
         self.n_pages = max(1, pages_for(int(max_tokens)))
         self.dtype = dtype
         self.device = device
@@ -162,7 +192,7 @@ class Cache:
     @property
     def kv_groups(self) -> List:
         """The groups that grow with their sequences in pages."""
-        return [g for g in self.groups if hasattr(g, "table")]
+        return [g for g in self.groups if getattr(g, "paged", False)]
 
     @property
     def state_groups(self) -> List:
@@ -240,8 +270,9 @@ class Cache:
 
     def block_tables(self, slots: Sequence[int]) -> Dict[int, List[List[int]]]:
         """Per paged group, per sequence of the step, its pages (a page given back behind a
-        window is never read; 0 stands in for it)."""
-        return {id(g): [[(p if p >= 0 else 0) for p in g.table.pages(s)] for s in slots] for g in self.kv_groups}
+        window is never read; 0 stands in for it).  The spare slot holds the spare page."""
+        return {id(g): [[g.spare_page] if s == self.spare_slot else [(p if p >= 0 else 0) for p in g.table.pages(s)]
+                        for s in slots] for g in self.kv_groups}
 
     def view(self, layer: int, block_tables: Dict[int, torch.Tensor]) -> LayerCacheView:
         v = LayerCacheView()

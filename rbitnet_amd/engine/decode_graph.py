@@ -9,6 +9,13 @@ temperatures, uniform numbers) from fixed device buffers.
 
 No memset is recorded into the graph (the buffers are written by a copy issued before
 each replay, outside the graph), and only this library's kernels run inside it.
+
+A batch whose sequences end one by one would need a capture for every size on the way down.
+Graphs are therefore captured for a ladder of sizes only (`graph_size`), and a batch runs in the
+graph of the next size up: the rows beyond its own are idle rows, each a sequence of length 0 in
+the cache's spare slot, whose token (id 0 at position 0) writes its key, value and state to the
+spare page and the spare state and reads nothing else.  A live row's result does not depend on the
+idle rows: every kernel of a step computes a row from that row's inputs alone.
 """
 from __future__ import annotations
 
@@ -17,6 +24,17 @@ from typing import Optional
 import torch
 
 from .context import StepBatch, StepContext, bucket_max_pages
+
+GRAPH_SIZES = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64)
+
+
+def graph_size(n_seqs: int) -> int:
+    """The size of the captured step that a batch of n sequences runs in: the next of 1, 2, 3, 4, 6,
+    8, 12, 16, 24, 32, 48, 64, and multiples of 32 beyond, so that at most a third of the rows idle."""
+    for size in GRAPH_SIZES:
+        if n_seqs <= size:
+            return size
+    return (int(n_seqs) + 31) // 32 * 32
 
 
 class DecodeGraph:
@@ -44,10 +62,14 @@ class DecodeGraph:
 
     def _fill(self, slots, tokens, temperatures, uniforms) -> None:
         cache = self.engine.cache
-        self.ctx.fill(StepBatch(slots=slots, past_lens=[cache.length(s) for s in slots],
-                                tokens=[[t] for t in tokens], rows=list(range(self.n_seqs)),
-                                block_tables=cache.block_tables(slots), temperatures=temperatures,
-                                uniforms=uniforms))
+        idle = self.n_seqs - len(slots)
+        past = [cache.length(s) for s in slots] + [0] * idle
+        slots = list(slots) + [cache.spare_slot] * idle
+        pad = lambda values: None if values is None else list(values) + [0.0] * idle
+        self.ctx.fill(StepBatch(slots=slots, past_lens=past,
+                                tokens=[[t] for t in tokens] + [[0]] * idle, rows=list(range(self.n_seqs)),
+                                block_tables=cache.block_tables(slots), temperatures=pad(temperatures),
+                                uniforms=pad(uniforms)))
 
     def _launch(self) -> None:
         eng, c = self.engine, self.ctx
@@ -55,8 +77,13 @@ class DecodeGraph:
         eng.lib.sample(self.logits, c.temperature, c.uniform, self.tokens_out)
 
     def run(self, slots, tokens, temperatures=None, uniforms=None) -> list:
+        """The step for these sequences (at most as many as the graph was made for); returns their
+        next tokens.  `logits`/`first_logits` hold a row per row of the graph, the live ones first."""
         eng = self.engine
-        q = [1] * self.n_seqs
+        n = len(slots)
+        if not 1 <= n <= self.n_seqs:
+            raise ValueError(f"a captured step for {self.n_seqs} sequences cannot run {n}")
+        q = [1] * n
         eng.cache.reserve(slots, q)
         self._fill(slots, tokens, temperatures, uniforms)
         if self.graph is None:
@@ -70,7 +97,7 @@ class DecodeGraph:
                 self._launch()
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()
-            out = self.tokens_out.tolist()
+            out = self.tokens_out.tolist()[:n]
             first_logits = self.logits.clone()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
@@ -81,6 +108,6 @@ class DecodeGraph:
             return out
         self.first_logits = None
         self.graph.replay()
-        out = self.tokens_out.tolist()
+        out = self.tokens_out.tolist()[:n]
         eng.cache.commit(slots, q)
         return out

@@ -56,7 +56,7 @@ class Engine:
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0}
         # per-kernel timers need every launch on its own
         self.use_graphs = bool(model.graph_safe) and getattr(self.lib, "times", None) is None
-        # (sequences, split bucket) -> DecodeGraph, least recently used first
+        # (rows of the captured step, split bucket) -> DecodeGraph, least recently used first
         self._graphs: "OrderedDict[Tuple[int, int], Any]" = OrderedDict()
         # float32 [sequences, vocab] of the last `decode_step`, valid until the next one
         self.last_decode_logits: Optional[torch.Tensor] = None
@@ -213,8 +213,9 @@ class Engine:
 
     def decode_step(self, slots: Sequence[int], tokens: Sequence[int], temperatures=None, uniforms=None) -> list:
         """One token per sequence in, the next token per sequence out: a step and the
-        sampling of its logits, replayed as a HIP graph per batch size (see
-        decode_graph.py); `use_graphs = False` runs the same kernels launch by launch."""
+        sampling of its logits, replayed as a HIP graph (captured for a ladder of batch sizes, a
+        batch running in the next size up with idle rows, see decode_graph.py);
+        `use_graphs = False` runs the same kernels launch by launch."""
         slots = [int(s) for s in slots]
         tokens = [int(t) for t in tokens]
         vocab = self.spec.vocab_size
@@ -227,23 +228,23 @@ class Engine:
             logits = self.step([(s, [t]) for s, t in zip(slots, tokens)], "last")
             self.last_decode_logits = logits
             return self.sampler.sample(logits, temperatures, uniforms)
-        from .decode_graph import DecodeGraph
+        from .decode_graph import DecodeGraph, graph_size
         n = len(slots)
-        key = (n, split_bucket(max(self.cache.length(s) for s in slots) + 1))
+        key = (graph_size(n), split_bucket(max(self.cache.length(s) for s in slots) + 1))
         if key not in self._graphs:
             if len(self._graphs) >= MAX_DECODE_GRAPHS:
                 self._graphs.popitem(last=False)           # the least recently used
-            self._graphs[key] = DecodeGraph(self, n, key[1])
+            self._graphs[key] = DecodeGraph(self, key[0], key[1])
         self._graphs.move_to_end(key)
         graph = self._graphs[key]
         out = graph.run(slots, tokens, temperatures, uniforms)
-        self.last_decode_logits = graph.logits if graph.first_logits is None else graph.first_logits
+        self.last_decode_logits = (graph.logits if graph.first_logits is None else graph.first_logits)[:n]
         self.stats["steps"] += 1
         self.stats["decode_tokens"] += n
         return out
 
     # ------------------------------------------------------------------ generation
-    def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 256, temperature: float = 0.7,
+    def generate(self, prompts: Sequence[Sequence[int]], max_tokens: Union[int, Sequence[int]] = 256, temperature: float = 0.7,
                  seed: int = 0, stop_token_ids: Optional[Sequence[int]] = None):
         from .generate import generate
         return generate(self, prompts, max_tokens=max_tokens, temperature=temperature, seed=seed,

@@ -21,7 +21,7 @@ loop counts tokens and leaves to the cache how it stores them.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Callable, List, Optional, Sequence
+from typing import Callable, List, Optional, Sequence, Union
 
 from ..errors import InferenceError
 from ..sampling.sampler import uniform
@@ -38,7 +38,7 @@ class GenerationResult:
 class _Running:
     index: int                       # position of the request in the caller's list
     slot: int
-    budget: int                      # new tokens it may still emit
+    budget: int                      # new tokens it may emit in all
     room: int                        # tokens the sequence may still hold
     result: GenerationResult = None
 
@@ -56,16 +56,17 @@ def decide(token: int, emitted: int, max_tokens: int, room_after: int, stop_ids)
     return None
 
 
-def plan_batches(prompt_lens: Sequence[int], max_tokens: int, max_batch: int, max_seq_len: int,
+def plan_batches(prompt_lens: Sequence[int], max_tokens, max_batch: int, max_seq_len: int,
                  capacity: int, needed: Callable[[int], int] = lambda n: n) -> List[List[int]]:
     """Requests in order, cut into batches that fit the slots and the cache: a request counts
-    with the most tokens it can come to hold, `needed(n)` being what n tokens take of the
-    cache's `capacity`."""
+    with the most tokens it can come to hold (max_tokens: one number, or one per request),
+    `needed(n)` being what n tokens take of the cache's `capacity`."""
     batches: List[List[int]] = []
     cur: List[int] = []
     used = 0
     for i, n in enumerate(prompt_lens):
-        need = needed(min(n + max_tokens, max_seq_len))
+        new = max_tokens if isinstance(max_tokens, int) else max_tokens[i]
+        need = needed(min(n + max(0, int(new)), max_seq_len))
         if need > capacity:
             need = capacity               # it will end with "context" when the cache is full
         if cur and (len(cur) >= max_batch or used + need > capacity):
@@ -78,10 +79,12 @@ def plan_batches(prompt_lens: Sequence[int], max_tokens: int, max_batch: int, ma
     return batches
 
 
-def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 256, temperature: float = 0.7,
-             seed: int = 0, stop_token_ids: Optional[Sequence[int]] = None) -> List[GenerationResult]:
+def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: Union[int, Sequence[int]] = 256,
+             temperature: float = 0.7, seed: int = 0,
+             stop_token_ids: Optional[Sequence[int]] = None) -> List[GenerationResult]:
     """Defaults as the reference's request fields: max_tokens 256, temperature 0.7
-    (crates/bitnet-server/src/lib.rs:317, :358)."""
+    (crates/bitnet-server/src/lib.rs:317, :358).  max_tokens may be one number per request, as
+    every request of the reference carries its own."""
     stop_ids = set(engine.spec.stop_token_ids) | set(int(t) for t in (stop_token_ids or ()))
     bos = getattr(engine.spec, "bos_token_id", None)
     prompts = [list(p) for p in prompts]
@@ -93,23 +96,31 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 256, te
         if len(prompts[i]) > engine.max_seq_len:
             raise InferenceError(f"request {i}: prompt of {len(prompts[i])} tokens exceeds max_seq {engine.max_seq_len}")
     results = [GenerationResult(prompt_tokens=len(p)) for p in prompts]
-    if max_tokens <= 0:
-        for r in results:
-            r.finish_reason = "length"
+    if isinstance(max_tokens, int):
+        limits = [int(max_tokens)] * len(prompts)
+    else:
+        limits = [int(m) for m in max_tokens]
+        if len(limits) != len(prompts):
+            raise InferenceError(f"{len(limits)} values of max_tokens for {len(prompts)} requests")
+    order = [i for i in range(len(prompts)) if limits[i] > 0]
+    for i in range(len(prompts)):
+        if limits[i] <= 0:
+            results[i].finish_reason = "length"
+    if not order:
         return results
     cache = engine.cache
     capacity = cache.token_capacity()
     for i, p in enumerate(prompts):
         if cache.tokens_needed(len(p)) > capacity:
             raise InferenceError(f"request {i}: prompt of {len(p)} tokens does not fit the cache")
-    batches = plan_batches([len(p) for p in prompts], max_tokens, engine.max_batch, engine.max_seq_len, capacity,
-                           cache.tokens_needed)
+    batches = plan_batches([len(prompts[i]) for i in order], [limits[i] for i in order], engine.max_batch,
+                           engine.max_seq_len, capacity, cache.tokens_needed)
 
     for batch in batches:
         running: List[_Running] = []
-        for i in batch:
+        for i in (order[j] for j in batch):
             slot = engine.alloc_slot()
-            running.append(_Running(index=i, slot=slot, budget=max_tokens,
+            running.append(_Running(index=i, slot=slot, budget=limits[i],
                                     room=engine.max_seq_len - len(prompts[i]), result=results[i]))
         try:
             logits = engine.step([(r.slot, prompts[r.index]) for r in running], "last")
@@ -120,7 +131,7 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 256, te
                 survivors: List[_Running] = []
                 feed: List[int] = []
                 for r, tok in zip(running, tokens):
-                    verdict = decide(tok, len(r.result.tokens), max_tokens, r.room - 1, stop_ids)
+                    verdict = decide(tok, len(r.result.tokens), r.budget, r.room - 1, stop_ids)
                     if verdict != "stop":
                         r.result.tokens.append(int(tok))
                         r.room -= 1

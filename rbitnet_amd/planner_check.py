@@ -27,30 +27,55 @@ def products(cfg: Dict) -> List[Tuple[str, int, int, int]]:
     return [("qkv", (hq + 2 * hk) * d, e, 0), ("o", e, hq * d, 0), ("gate_up", 2 * f, e, 1), ("down", e, f, 0)]
 
 
-def _time(lib, torch, fn, reps: int) -> float:
-    fn(0)
-    torch.cuda.synchronize()
-    best = float("inf")
-    for _ in range(3):
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for i in range(reps):
-            fn(i)
-        end.record()
-        torch.cuda.synchronize()
-        best = min(best, start.elapsed_time(end) * 1e3 / reps)
+def _time_all(torch, candidates, run, reps: int, rounds: int = 5) -> List[float]:
+    """The least time in microseconds of every candidate (a function that sets the choice up) over
+    `rounds` rounds in which the candidates take turns, so that a drift of the clock or of the
+    memory's state touches all of them alike; a candidate that the kernels refuse gets inf."""
+    from .errors import KernelError
+    best = [float("inf")] * len(candidates)
+    alive = [True] * len(candidates)
+    for _ in range(rounds):
+        for j, setup in enumerate(candidates):
+            if not alive[j]:
+                continue
+            setup()
+            try:
+                run(0)
+            except KernelError:
+                alive[j] = False
+                continue
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for i in range(reps):
+                run(i + 1)
+            end.record()
+            torch.cuda.synchronize()
+            best[j] = min(best[j], start.elapsed_time(end) * 1e3 / reps)
     return best
 
 
-def sweep(models: Sequence[Tuple[str, Dict]], token_counts: Sequence[int], out=sys.stdout) -> float:
-    """Prints the table; returns the worst ratio of the planner's time to the best forced time."""
+def sweep(models: Sequence[Tuple[str, Dict]], token_counts: Sequence[int], out=sys.stdout, detail=None) -> float:
+    """Prints the table; returns the worst ratio of the planner's time to the best forced time.
+    detail: a file that gets one line per product with the time of every candidate."""
     import torch
     from .csrc.lib import kernels
-    from .errors import KernelError
     lib = kernels()
     L = lib._lib
     dev = torch.device("cuda:0")
     worst = 1.0
+
+    def reset():
+        L.rb_tune_tiles(0, 0)
+        L.rb_tune(0, 0)
+        L.rb_tune_use_resident(1)
+        L.rb_tune_use_stream(1)
+
+    def tile(cfg, parts):
+        return lambda: (reset(), L.rb_tune_tiles(cfg, parts))
+
+    def skinny(r, waves):
+        return lambda: (reset(), L.rb_tune_use_resident(0), L.rb_tune(r, waves))
+
     print("| shape | product | rows x K | tokens | planner | us | best forced | us | planner / best |", file=out)
     print("|---|---|---|---|---|---|---|---|---|", file=out)
     for label, cfg in models:
@@ -62,55 +87,44 @@ def sweep(models: Sequence[Tuple[str, Dict]], token_counts: Sequence[int], out=s
                 c = torch.empty((m, n // 2 if epi else n), dtype=torch.bfloat16 if epi else torch.float32, device=dev)
                 reps = max(4, min(40, int(2e4 / max(1.0, m * n * k * 2 / 1e9))))
                 run = lambda i: lib.gemm_bf16(a, ws[i % copies], c, epi, w_frag=True)
+                reset()
+                plan = int(L.rb_tune_plan(m, n, k, epi))
+                chosen = f"tile {plan // 100} x {plan % 100}" if plan else "few-token kernels"
+                names, setups = ["planner"], [reset]
+                if m > 16:
+                    for cfg_id in (SMALL_TILE_CFGS if m <= 64 else TILE_CFGS):
+                        if cfg_id == 13 and k % 128:
+                            continue
+                        for parts in ((1,) if epi else ((1, 2, 4, 8) if m > 512 else range(1, 9))):
+                            if (k // 64) % parts or k // 64 // parts < 4:
+                                continue
+                            names.append(f"tile {cfg_id} x {parts}")
+                            setups.append(tile(cfg_id, parts))
+                    if m <= 64:
+                        names.append("few-token kernels")
+                        setups.append(lambda: (reset(), L.rb_tune_use_stream(0)))
+                else:
+                    names.append("resident")
+                    setups.append(lambda: (reset(), L.rb_tune_use_resident(2)))
+                    for r in (1, 2, 4):
+                        if epi and r == 1:
+                            continue
+                        for waves in (4, 8):
+                            names.append(f"skinny {r} tiles a wave, {waves} waves")
+                            setups.append(skinny(r, waves))
                 try:
-                    L.rb_tune_tiles(0, 0)
-                    L.rb_tune(0, 0)
-                    L.rb_tune_use_resident(1)
-                    L.rb_tune_use_stream(1)
-                    plan = int(L.rb_tune_plan(m, n, k, epi))
-                    chosen = f"tile {plan // 100} x {plan % 100}" if plan else "few-token kernels"
-                    t_plan = _time(lib, torch, run, reps)
-                    forced: List[Tuple[float, str]] = []
-                    if m > 16:
-                        for tile in (SMALL_TILE_CFGS if m <= 64 else TILE_CFGS):
-                            if tile == 13 and k % 128:
-                                continue
-                            for parts in ((1,) if epi else ((1, 2, 4, 8) if m > 512 else range(1, 9))):
-                                if (k // 64) % parts or k // 64 // parts < 4:
-                                    continue
-                                L.rb_tune_tiles(tile, parts)
-                                try:
-                                    forced.append((_time(lib, torch, run, reps), f"tile {tile} x {parts}"))
-                                except KernelError:
-                                    pass                    # a tile that does not take this many slices
-                        L.rb_tune_tiles(0, 0)
-                        if m <= 64:
-                            L.rb_tune_use_stream(0)
-                            forced.append((_time(lib, torch, run, reps), "few-token kernels"))
-                            L.rb_tune_use_stream(1)
-                    else:
-                        for resident in (0, 2):
-                            L.rb_tune_use_resident(resident)
-                            if resident:
-                                forced.append((_time(lib, torch, run, reps), "resident"))
-                                continue
-                            for r in (1, 2, 4):
-                                if epi and r == 1:
-                                    continue
-                                for waves in (4, 8):
-                                    L.rb_tune(r, waves)
-                                    forced.append((_time(lib, torch, run, reps), f"skinny {r} tiles a wave, {waves} waves"))
-                            L.rb_tune(0, 0)
+                    times = _time_all(torch, setups, run, reps)
                 finally:
-                    L.rb_tune_tiles(0, 0)
-                    L.rb_tune(0, 0)
-                    L.rb_tune_use_resident(1)
-                    L.rb_tune_use_stream(1)
-                t_best, which = min(forced)
+                    reset()
+                t_plan = times[0]
+                t_best, which = min(zip(times[1:], names[1:]))
                 ratio = t_plan / t_best
                 worst = max(worst, ratio)
                 print(f"| {label} | {name} | {n} x {k} | {m} | {chosen} | {t_plan:.1f} | {which} | {t_best:.1f} | "
                       f"{ratio:.3f} |", file=out, flush=True)
+                if detail is not None:
+                    print(f"{label}; {name} {n} x {k}; {m} tokens; planner: {chosen}; " +
+                          "; ".join(f"{nm}: {t:.1f}" for nm, t in zip(names, times)), file=detail, flush=True)
             del ws
             torch.cuda.empty_cache()
     print(f"\nworst planner / best: {worst:.3f}", file=out)

@@ -33,7 +33,7 @@ def test_pages_follow_lengths_and_come_back():
     c = _cache()
     assert c.n_pages == 10 and len(c.kv_groups) == 1
     g = c.kv_groups[0]
-    assert g.k.shape == (3, 10, 2, PAGE_SIZE, 8)
+    assert g.k.shape == (3, 10 + 1, 2, PAGE_SIZE, 8)           # and the spare page
     a, b = c.alloc_slot(), c.alloc_slot()
     c.reserve([a, b], [65, 1])
     assert len(g.table.pages(a)) == 2 and len(g.table.pages(b)) == 1
@@ -108,7 +108,7 @@ def test_groups_by_need_and_readers():
     full = kv(0)[0]
     assert full.layers == [0, 3] and kv(3) == (full, 1)
     assert kv(2) == kv(1)                            # layer 2 reads layer 1's keys and values
-    assert kv(4)[0].k.shape == (1, 8, 1, PAGE_SIZE, 16)
+    assert kv(4)[0].k.shape == (1, 8 + 1, 1, PAGE_SIZE, 16)
     with pytest.raises(CacheError, match="keeps none"):
         Cache([None, CacheRequest("kv", heads=1, head_dim=8)], 1, 64, torch.float32, "cpu", readers={1: 0})
 
@@ -136,7 +136,7 @@ def test_state_is_reset_when_a_slot_is_handed_out():
     c = Cache(reqs, 2, 64, torch.float32, "cpu")
     s = c.alloc_slot()
     st = c.view(0, {}).state
-    assert st.shape == (2, 4) and torch.all(st[s] == 2.0)
+    assert st.shape == (2 + 1, 4) and torch.all(st[s] == 2.0)         # two slots and the spare one
     st[s] += 5
     c.free_slot(s)
     assert c.alloc_slot() == s and torch.all(c.view(0, {}).state[s] == 2.0)

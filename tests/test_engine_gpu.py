@@ -227,13 +227,13 @@ def test_cache_for_a_configuration_with_a_very_long_context(tmp_path, monkeypatc
     folder = rbitnet_amd.write_random_model(str(tmp_path / "m"), cfg, seed=0, std=0.1)
     per_token = 2 * cfg["num_hidden_layers"] * cfg["num_key_value_heads"] * 16 * 2        # k and v, bfloat16
     eng = rbitnet_amd.Engine.load_path(folder)
-    assert eng.max_seq_len == 131072 and eng.cache.bytes() == 8 * 131072 * per_token
+    assert eng.max_seq_len == 131072 and eng.cache.bytes() == (8 * 131072 + 64) * per_token      # and the spare page
     del eng
     real = torch.cuda.mem_get_info
     monkeypatch.setattr(torch.cuda, "mem_get_info", lambda *a: (1 << 20, real(*a)[1]))    # 1 MiB is free
     eng = rbitnet_amd.Engine.load_path(folder)
     fits = int((1 << 20) * 0.9) // per_token // 64 * 64
-    assert eng.cache.bytes() == fits * per_token and eng.cache.token_capacity() == fits
+    assert eng.cache.bytes() == (fits + 64) * per_token and eng.cache.token_capacity() == fits
     assert "sized to the" in capfd.readouterr().err
     (r,) = eng.generate([tokens_for("A", fits - 10, 1)], max_tokens=100, temperature=0.0, stop_token_ids=[])
     assert r.finish_reason == "context" and len(r.tokens) == 11       # ten run, the last is only emitted

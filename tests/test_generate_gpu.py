@@ -239,3 +239,55 @@ def test_graph_decode_equals_launch_by_launch(dtype):
     seq0 = prompts[0] + [t[0] for t in tok_g[:-1]]
     last = [h for h in outs[0] if isinstance(h, torch.Tensor)][-1]
     assert max_err(last[0:1], plain_logits(name, tuple(seq0))[-1:]) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_idle_rows_of_a_captured_step_touch_no_live_sequence(name, dtype):
+    """Captured steps exist for a ladder of sizes; a batch of 5 runs in 6 rows, then, as sequences
+    leave one by one, in 4, 3, 2 and 1.  Between two steps the cache may change at the live
+    sequences' new positions and in the spare page and nowhere else; every live row's logits
+    match the plain implementation; the state of the free lists stays sound."""
+    from rbitnet_amd.engine.decode_graph import graph_size
+    assert [graph_size(n) for n in (1, 2, 3, 4, 5, 6, 7, 9, 13, 17, 20, 33, 49, 64, 65, 97, 200)] == \
+        [1, 2, 3, 4, 6, 6, 8, 12, 16, 24, 24, 48, 64, 64, 96, 128, 224]
+    lengths = [70, 5, 64, 33, 12]
+    reqs = [tokens_for(name, n + 9, 80 + i) for i, n in enumerate(lengths)]
+    eng = _engine(name, dtype, max_batch=5, max_tokens=64 * 8)
+    assert eng.use_graphs
+    groups = eng.cache.kv_groups
+    for g in groups:
+        g.k.fill_(3.0)
+        g.v.fill_(3.0)
+    slots = [eng.alloc_slot() for _ in reqs]
+    eng.step([(s, r[:n]) for s, r, n in zip(slots, reqs, lengths)], [[] for _ in reqs])
+    live = list(range(len(reqs)))
+    sizes = []
+    for j in range(9):
+        before = [(g.k.clone(), g.v.clone()) for g in groups]
+        lens = [eng.cache.length(slots[i]) for i in live]
+        eng.cache.reserve([slots[i] for i in live], [1] * len(live))      # so that the pages of this step are known here
+        tables = eng.cache.block_tables([slots[i] for i in live])
+        eng.decode_step([slots[i] for i in live], [reqs[i][lengths[i] + j] for i in live])
+        sizes.append(graph_size(len(live)))
+        got = eng.last_decode_logits.float().cpu()
+        assert got.shape[0] == len(live)
+        for row, i in enumerate(live):
+            want = plain_logits(name, tuple(reqs[i]))[lengths[i] + j]
+            assert max_err(got[row:row + 1], want[None]) < TOL[dtype], (j, i)
+        for g, (k0, v0) in zip(groups, before):
+            allowed = torch.zeros(g.k.shape[1], 64, dtype=torch.bool, device=g.k.device)
+            allowed[g.spare_page] = True
+            for pages, n in zip(tables[id(g)], lens):
+                allowed[pages[n // 64], n % 64] = True
+            for new, old in ((g.k, k0), (g.v, v0)):
+                changed = (new != old).any(dim=4).any(dim=2).any(dim=0)        # [pages, 64]
+                assert not bool((changed & ~allowed).any()), f"step {j}: a position outside the step's own was written"
+        if j in (1, 3, 5, 6):                                       # a sequence leaves: 5, 4, 3, 2, 1
+            eng.free_slot(slots[live.pop(1 if len(live) > 1 else 0)])
+    assert sizes == [6, 6, 4, 4, 3, 3, 2, 1, 1]
+    assert sorted(n for n, _ in eng._graphs) == [1, 2, 3, 4, 6]
+    for i in live:
+        eng.free_slot(slots[i])
+    eng.cache.check()
+    assert eng.cache.slots.n_held == 0

@@ -73,6 +73,22 @@ def test_max_tokens_and_no_wasted_step():
     assert generate(eng, [[1]], max_tokens=0)[0].finish_reason == "length"
 
 
+def test_a_limit_of_its_own_for_every_request():
+    """max_tokens as a list: every request ends at its own limit, a request with none runs no step,
+    and the cache is planned with each request's own growth."""
+    eng = ScriptedEngine(max_batch=3)
+    rs = generate(eng, [[10], [1], [12], [2]], max_tokens=[3, 0, 1, 5], temperature=0.0, stop_token_ids=[])
+    assert [r.tokens for r in rs] == [[11, 12, 13], [], [13], [3, 4, 5, 6, 7]]
+    assert [r.finish_reason for r in rs] == ["length"] * 4
+    assert eng.steps[0] == [(0, [10]), (1, [12]), (2, [2])]          # the request without a budget holds no slot
+    assert eng.steps[1] == [(0, [11]), (2, [3])]                      # the one with a single token has left
+    assert [len(s) for s in eng.steps] == [3, 2, 2, 1, 1]
+    with pytest.raises(InferenceError, match="values of max_tokens"):
+        generate(eng, [[1], [2]], max_tokens=[3])
+    assert plan_batches([10, 10, 10], [100, 20, 20], 8, 1000, 192, lambda n: (n + 63) // 64 * 64) == [[0, 1], [2]]
+    assert eng.cache.slots.n_held == 0
+
+
 def test_unequal_batch_shorter_requests_end_earlier_and_slots_are_reused():
     eng = ScriptedEngine(max_batch=2)
     prompts = [[7], [1, 2], [8], [0]]

@@ -234,7 +234,7 @@ def test_toy_mixer_and_mixed_layers(dtype, tol):
     tensors = dict(random_tensors(expected, seed=4, std=0.15, norm_std=0.05, dtype=torch.bfloat16))
     eng = rbitnet_amd.Engine.from_spec(spec, tensors, dtype=dtype, max_tokens=64 * 12, max_batch=3)
     assert len(eng.cache.kv_groups) == 1 and len(eng.cache.state_groups) == 1
-    assert eng.cache.state_groups[0].data.shape[0] == 2            # two runs of layer 1, two states
+    assert eng.cache.state_groups[0].data.shape[:2] == (2, 3 + 1)  # two runs of layer 1, two states; 3 slots and the spare one
     g = torch.Generator().manual_seed(8)
     seqs = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in (130, 9, 70)]
     want = [_plain_toy_model(spec, tensors, s) for s in seqs]
@@ -579,20 +579,20 @@ def test_embedding_with_a_scale_and_capped_head_registered_from_here(dtype, tol)
     from rbitnet_amd.weights import random_tensors
     register_embedding("scaled_table", ScaledTable)
     register_head("capped", CappedHead)
-    hidden, vocab, scale, cap = 64, 75, 3.5, 2.0
+    hidden, vocab, scale = 64, 75, 3.5
     norm = PartSpec("rmsnorm", {"size": hidden, "eps": 1e-5})
     att = _attention_params(4, 2, 16, window=None)
     layers = [LayerSpec(f"blocks.{i}", "prenorm", PartSpec("attention", att), PartSpec("swiglu", {"intermediate_size": 48}),
                         norm, norm) for i in range(2)]
-    spec = ModelSpec(architecture="ToyForTests", hidden_size=hidden, vocab_size=vocab, max_positions=256, layers=layers,
-                     embedding=PartSpec("scaled_table", {"name": "tokens.weight", "vocab_size": vocab, "scale": scale}),
-                     head=PartSpec("capped", {"norm": norm, "vocab_size": vocab, "cap": cap}))
-    expected = expected_tensors(spec)
+    make_spec = lambda cap: ModelSpec(
+        architecture="ToyForTests", hidden_size=hidden, vocab_size=vocab, max_positions=256, layers=layers,
+        embedding=PartSpec("scaled_table", {"name": "tokens.weight", "vocab_size": vocab, "scale": scale}),
+        head=PartSpec("capped", {"norm": norm, "vocab_size": vocab, "cap": cap}))
+    expected = expected_tensors(make_spec(1.0))
     assert {"tokens.weight", "out.norm.weight", "out.proj.weight"} <= set(expected)
     tensors = dict(random_tensors(expected, seed=9, std=0.15, norm_std=0.05, dtype=torch.bfloat16))
-    tensors["out.proj.weight"] = tensors["out.proj.weight"] * 6          # logits large enough for the cap to bend them
 
-    def plain(tokens):
+    def plain(tokens, cap):
         # the plain Llama layers between the test's own ends
         w = {k: v.double().cpu() for k, v in tensors.items()}
         x = P.embedding(w["tokens.weight"], tokens) * scale
@@ -607,14 +607,15 @@ def test_embedding_with_a_scale_and_capped_head_registered_from_here(dtype, tol)
             x = x + P.swiglu(h2, w[f"{pre}.mlp.gate_proj.weight"], w[f"{pre}.mlp.up_proj.weight"],
                              w[f"{pre}.mlp.down_proj.weight"])
         z = P.linear(P.rmsnorm(x, w["out.norm.weight"], 1e-5), w["out.proj.weight"])
-        return cap * torch.tanh(z / cap)
+        return z if cap is None else cap * torch.tanh(z / cap)
 
-    eng = rbitnet_amd.Engine.from_spec(spec, tensors, dtype=dtype, max_tokens=64 * 4, max_batch=2)
-    assert eng.use_graphs
     g = torch.Generator().manual_seed(12)
     seqs = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in (70, 12)]
-    want = [plain(s) for s in seqs]
-    assert float(want[0].abs().max()) > 0.9 * cap                         # the cap does bend them
+    cap = float(plain(seqs[0], None).abs().max()) / 2                     # a cap that bends the large logits
+    want = [plain(s, cap) for s in seqs]
+    assert float(want[0].abs().max()) > 0.9 * cap
+    eng = rbitnet_amd.Engine.from_spec(make_spec(cap), tensors, dtype=dtype, max_tokens=64 * 4, max_batch=2)
+    assert eng.use_graphs
     slots = [eng.alloc_slot() for _ in seqs]
     cut = [len(s) - 4 for s in seqs]
     logits = eng.step([(sl, s[:c]) for sl, s, c in zip(slots, seqs, cut)], "all")
