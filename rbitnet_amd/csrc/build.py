@@ -154,5 +154,79 @@ def ensure_built(verbose: bool = True) -> str:
         raise
 
 
+# ---------------------------------------------------------------- the plain C++ twins (no GPU)
+PLAIN_LIB_NAME = "librbitnet_plain.so"
+PLAIN_SELFTEST_NAME = "plain_selftest"
+PLAIN_SOURCES = ["plain.cpp", "plain.h", "plain_selftest.cpp"]
+PLAIN_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Werror"]
+SANITIZE = ["-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-fno-omit-frame-pointer", "-static-libasan",
+            "-static-libubsan", "-g"]
+
+
+def _host_compiler() -> str:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++")):
+        if cand and os.path.isfile(cand):
+            return cand
+    raise RuntimeError("no host C++ compiler found (looked at $CXX, g++, c++, clang++)")
+
+
+def _plain_digest() -> str:
+    h = hashlib.sha256()
+    for name in PLAIN_SOURCES:
+        with open(os.path.join(HERE, name), "rb") as f:
+            h.update(name.encode())
+            h.update(f.read())
+    h.update(" ".join(PLAIN_FLAGS + SANITIZE).encode())
+    return h.hexdigest()[:16]
+
+
+def _plain_built(name: str) -> Optional[str]:
+    digest = _plain_digest()
+    for folder in _candidate_dirs():
+        path = os.path.join(folder, name)
+        if os.path.isfile(path) and os.path.isfile(path + ".stamp"):
+            with open(path + ".stamp") as f:
+                if f.read().strip() == digest:
+                    return path
+    return None
+
+
+def _compile_host(args: List[str], out_name: str) -> str:
+    out_dir = next((d for d in _candidate_dirs() if _writable(d)), None)
+    if out_dir is None:
+        raise RuntimeError("no writable folder for the built twins")
+    out = os.path.join(out_dir, out_name)
+    tmp = out + f".tmp{os.getpid()}"
+    r = subprocess.run([_host_compiler()] + args + ["-o", tmp], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"compiling {out_name} failed:\n{r.stderr[-4000:]}")
+    os.replace(tmp, out)
+    with open(out + ".stamp", "w") as f:
+        f.write(_plain_digest())
+    return out
+
+
+def build_plain(force: bool = False) -> str:
+    """The twins as a shared library for ctypes (host compiler, no GPU code).  Returns its path."""
+    if not force:
+        lib = _plain_built(PLAIN_LIB_NAME)
+        if lib:
+            return lib
+    return _compile_host(PLAIN_FLAGS + ["-shared", os.path.join(HERE, "plain.cpp")], PLAIN_LIB_NAME)
+
+
+def build_plain_selftest(force: bool = False) -> str:
+    """The twins and their self-test as one program under the address and undefined-behaviour
+    sanitizers (their run-time parts linked in statically, so that nothing has to be preloaded)."""
+    if not force:
+        exe = _plain_built(PLAIN_SELFTEST_NAME)
+        if exe:
+            return exe
+    return _compile_host(PLAIN_FLAGS + SANITIZE + [os.path.join(HERE, "plain.cpp"), os.path.join(HERE, "plain_selftest.cpp")],
+                         PLAIN_SELFTEST_NAME)
+
+
 if __name__ == "__main__":
     print(build(force=True))
+    print(build_plain(force=True))
+    print(build_plain_selftest(force=True))

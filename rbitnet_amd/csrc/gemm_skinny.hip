@@ -404,8 +404,11 @@ static int dispatch_skinny(const GemmTokens& x, const bf16_t* w, void* c, const 
   // 10240 rows at K = 8192 with one token: R = 1 35 us, R = 2 42; R = 4 takes 31 us by itself (160
   // workgroups), but the decode step of that shape is no faster with it (+0.3 % at batch 1, +0.5 % at
   // 8, -1.1 % at 16, each the mean of four runs in alternating order), so it is not taken.
+  // Between K = 4096 and 8192 the same estimate holds: 15,360 rows at K = 5120 with 16 tokens 26.6 us
+  // with R = 4 against 33.6 with R = 1 (8 tokens: 26.4 against 27.5, one token 26.9 against 26.5),
+  // 5,120 rows 13.6 with R = 2 against 16.8 (8 tokens: 12.1 against 13.4).
   int r = 1;
-  if (k >= 8192) {
+  if (k > 4096) {
     double best = 0.0;
     const long long cus = rb_compute_units();
     for (int cand = (EPI == 1 ? 2 : 1); cand <= 4; cand *= 2) {

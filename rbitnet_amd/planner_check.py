@@ -67,6 +67,7 @@ def sweep(models: Sequence[Tuple[str, Dict]], token_counts: Sequence[int], out=s
     def reset():
         L.rb_tune_tiles(0, 0)
         L.rb_tune(0, 0)
+        L.rb_tune_resident(0)
         L.rb_tune_use_resident(1)
         L.rb_tune_use_stream(1)
 
@@ -104,8 +105,9 @@ def sweep(models: Sequence[Tuple[str, Dict]], token_counts: Sequence[int], out=s
                         names.append("few-token kernels")
                         setups.append(lambda: (reset(), L.rb_tune_use_stream(0)))
                 else:
-                    names.append("resident")
-                    setups.append(lambda: (reset(), L.rb_tune_use_resident(2)))
+                    for tiles in (0, 1, 2, 4, 8):
+                        names.append("resident" if tiles == 0 else f"resident, {tiles} row tiles a workgroup")
+                        setups.append(lambda tiles=tiles: (reset(), L.rb_tune_use_resident(2), L.rb_tune_resident(tiles)))
                     for r in (1, 2, 4):
                         if epi and r == 1:
                             continue
