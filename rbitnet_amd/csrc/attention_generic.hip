@@ -120,6 +120,8 @@ extern "C" int rb_attention_generic(const void* q, const void* k_pages, const vo
                                     const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table,
                                     int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                                     float scale, int window, void* stream) {
+  RB_RECORDED(rb_attention_generic(q, k_pages, v_pages, out, dtype, tok_pos, tok_seq, block_table, bt_stride, n_tokens, n_heads,
+                                   n_kv_heads, head_dim, scale, window, stream));
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
              "rb_attention_generic: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
   RB_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= AG_MAX_D,

@@ -307,6 +307,8 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
                                          const int32_t* block_table, int bt_stride, int n_seqs, int max_q_len,
                                          int n_heads, int n_kv_heads, int head_dim, float scale, int window,
                                          void* stream) {
+  RB_RECORDED(rb_attention_prefill_bf16(q, k_pages, v_pages, out, cu_seqlens, past_len, block_table, bt_stride, n_seqs,
+                                        max_q_len, n_heads, n_kv_heads, head_dim, scale, window, stream));
   RB_REQUIRE(n_seqs > 0 && max_q_len > 0, "rb_attention_prefill_bf16: empty batch");
   RB_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
              "rb_attention_prefill_bf16: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
@@ -1096,6 +1098,8 @@ extern "C" int rb_attention_decode_bf16(const void* q, const void* k_pages, cons
                                         const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
                                         int n_seqs, int n_heads, int n_kv_heads, int head_dim, float scale,
                                         int window, int n_splits, float* workspace, void* stream) {
+  RB_RECORDED(rb_attention_decode_bf16(q, k_pages, v_pages, out, tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads,
+                                       head_dim, scale, window, n_splits, workspace, stream));
   DecodeArgs a = {nullptr, (const bf16_t*)q, nullptr, nullptr, 0, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out,
                   tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, scale * LOG2E, window, n_splits,
                   workspace, 1, 0};
@@ -1108,6 +1112,9 @@ extern "C" int rb_attention_decode_fused_bf16(const float* qkv, int qkv_terms, l
                                               const int32_t* block_table, int bt_stride, int n_seqs, int n_heads,
                                               int n_kv_heads, int head_dim, float scale, int window, int n_splits,
                                               float* workspace, void* stream) {
+  RB_RECORDED(rb_attention_decode_fused_bf16(qkv, qkv_terms, qkv_term_stride, cos, sin, style, k_pages, v_pages, out, tok_pos,
+                                             block_table, bt_stride, n_seqs, n_heads, n_kv_heads, head_dim, scale, window,
+                                             n_splits, workspace, stream));
   RB_REQUIRE((cos == nullptr) == (sin == nullptr), "rb_attention_decode_fused_bf16: cos and sin tables go together");
   RB_REQUIRE(style == 0 || style == 1, "rb_attention_decode_fused_bf16: unknown pairing style %d", style);
   RB_REQUIRE(qkv_terms >= 1 && qkv_term_stride >= 0, "rb_attention_decode_fused_bf16: %d terms, %lld apart", qkv_terms,

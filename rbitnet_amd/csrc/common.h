@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <functional>
+
 #define RB_WAVE 64
 #define RB_PAGE 64            // tokens per cache page; attention tiles are one page of keys
 
@@ -34,6 +36,23 @@ enum RbDtype { RB_F32 = 0, RB_BF16 = 1 };
 // of workgroups is.  Every choice of a tile, a number of K slices or of splits that depends on
 // how a grid fills the GPU is an expression of this number, not of the 256 of an MI355X.
 int rb_compute_units(void);
+
+// ---------------------------------------------------------------- recorded steps (plan.hip)
+// While a plan records on the calling thread, every entry point that launches kernels notes its
+// own call (a closure over its arguments that takes the stream to launch on) before it does its
+// work, so that the same launches can be issued again from C++ without the caller's host code
+// between them.  RB_RECORDED(call) stands first in such an entry point, `call` being the entry
+// point's own call with its own parameter names, `stream` among them.  An entry point that
+// calls another one is recorded once, as itself.
+bool rb_plan_wants_call(void);
+void rb_plan_note(std::function<int(void*)> call);
+struct RbPlanScope {
+  RbPlanScope();
+  ~RbPlanScope();
+};
+#define RB_RECORDED(call)  \
+  RbPlanScope rb_plan_scope_; \
+  if (rb_plan_wants_call()) rb_plan_note([=](void* stream) -> int { return call; })
 
 // ---------------------------------------------------------------- bfloat16 storage
 struct bf16_t {

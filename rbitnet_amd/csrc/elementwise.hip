@@ -47,6 +47,7 @@ __global__ void embed_gather_kernel(const T* __restrict__ table, const int32_t* 
 
 extern "C" int rb_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* x, int n_tokens,
                                int width, void* stream) {
+  RB_RECORDED(rb_embed_gather(table, table_dtype, ids, x, n_tokens, width, stream));
   RB_REQUIRE(n_tokens >= 0 && width > 0, "rb_embed_gather: bad sizes %d x %d", n_tokens, width);
   if (n_tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
@@ -199,6 +200,7 @@ static bool launch_add_rmsnorm_vec(float* x, const float* delta, int n_terms, si
 extern "C" int rb_add_rmsnorm(float* x, const float* delta, int n_terms, long long term_stride_ll, const float* gain,
                               float eps, const int32_t* rows, int n_rows, int width, void* out, int out_dtype,
                               void* stream) {
+  RB_RECORDED(rb_add_rmsnorm(x, delta, n_terms, term_stride_ll, gain, eps, rows, n_rows, width, out, out_dtype, stream));
   RB_REQUIRE(n_rows >= 0 && width > 0, "rb_add_rmsnorm: bad sizes %d x %d", n_rows, width);
   RB_REQUIRE(!delta || (n_terms >= 1 && term_stride_ll >= 0), "rb_add_rmsnorm: %d terms, %lld apart", n_terms,
              term_stride_ll);
@@ -374,6 +376,8 @@ extern "C" int rb_rope_kv_write(const float* qkv, int qkv_terms, long long qkv_t
                                 void* k_pages, void* v_pages, int cache_dtype, const int32_t* tok_pos,
                                 const int32_t* tok_seq, const int32_t* block_table, int bt_stride, int n_tokens,
                                 int n_heads, int n_kv_heads, int head_dim, void* stream) {
+  RB_RECORDED(rb_rope_kv_write(qkv, qkv_terms, qkv_term_stride, cos, sin, style, q_out, k_pages, v_pages, cache_dtype,
+                               tok_pos, tok_seq, block_table, bt_stride, n_tokens, n_heads, n_kv_heads, head_dim, stream));
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0 && head_dim % 2 == 0,
              "rb_rope_kv_write: bad sizes T=%d Hq=%d Hk=%d D=%d", n_tokens, n_heads, n_kv_heads, head_dim);
   RB_REQUIRE(qkv_terms >= 1 && qkv_term_stride >= 0, "rb_rope_kv_write: %d terms, %lld apart", qkv_terms,
@@ -425,6 +429,7 @@ __global__ void swiglu_kernel(const float* __restrict__ gu, TO* __restrict__ out
 }
 
 extern "C" int rb_swiglu(const float* gu, void* out, int out_dtype, int n_rows, int ff, void* stream) {
+  RB_RECORDED(rb_swiglu(gu, out, out_dtype, n_rows, ff, stream));
   RB_REQUIRE(n_rows >= 0 && ff > 0, "rb_swiglu: bad sizes %d x %d", n_rows, ff);
   RB_REQUIRE(n_rows <= 65535 * 64, "rb_swiglu: too many rows %d", n_rows);
   if (n_rows == 0) return 0;

@@ -233,6 +233,7 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
 
 extern "C" int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dtype_out, int m, int n,
                                int k, void* stream) {
+  RB_RECORDED(rb_gemm_generic(a, w, c, dtype_in, dtype_out, m, n, k, stream));
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_generic: bad sizes M=%d N=%d K=%d", m, n, k);
   if (m == 0) return 0;
   hipStream_t s = (hipStream_t)stream;

@@ -40,6 +40,7 @@ static bool layout_ok(int w_layout, int n, int k) {
 
 extern "C" int rb_gemm_bf16(const void* a, const void* w, int w_layout, void* c, int dtype_out, int epilogue, int m,
                             int n, int k, float* workspace, void* stream) {
+  RB_RECORDED(rb_gemm_bf16(a, w, w_layout, c, dtype_out, epilogue, m, n, k, workspace, stream));
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_bf16: bad sizes M=%d N=%d K=%d", m, n, k);
   RB_REQUIRE(layout_ok(w_layout, n, k), "rb_gemm_bf16: W layout %d with N=%d K=%d (fragment-major needs N %% 16 == 0, K %% 64 == 0)",
              w_layout, n, k);
@@ -73,6 +74,7 @@ extern "C" int rb_gemm_bf16_terms_count(int m, int n, int k) {
 
 extern "C" int rb_gemm_bf16_terms(const void* a, const void* w, int w_layout, float* terms, int m, int n, int k,
                                   void* stream) {
+  RB_RECORDED(rb_gemm_bf16_terms(a, w, w_layout, terms, m, n, k, stream));
   const int p = rb_gemm_bf16_terms_count(m, n, k);
   if (p == 1) return rb_gemm_bf16(a, w, w_layout, terms, RB_F32, 0, m, n, k, nullptr, stream);
   RB_REQUIRE(layout_ok(w_layout, n, k), "rb_gemm_bf16_terms: W layout %d with N=%d K=%d", w_layout, n, k);
@@ -90,6 +92,8 @@ extern "C" int rb_gemm_bf16_few_ok(int m, int n, int k) {
 extern "C" int rb_gemm_bf16_few(const void* a, const float* squares_in, float eps, const int32_t* rows, const void* w,
                                 int w_layout, void* c, int dtype_out, int epilogue, const float* gain, void* gained,
                                 float* squares_out, int m, int n, int k, void* stream) {
+  RB_RECORDED(rb_gemm_bf16_few(a, squares_in, eps, rows, w, w_layout, c, dtype_out, epilogue, gain, gained, squares_out, m, n, k,
+                               stream));
   RB_REQUIRE(layout_ok(w_layout, n, k), "rb_gemm_bf16_few: W layout %d with N=%d K=%d", w_layout, n, k);
   RB_REQUIRE(rb_gemm_bf16_few_ok(m, n, k), "rb_gemm_bf16_few: M=%d N=%d K=%d is not for it (1..16 tokens, K %% 8 == 0)",
              m, n, k);

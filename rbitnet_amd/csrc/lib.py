@@ -150,6 +150,11 @@ class Kernels:
             fn = getattr(L, name)
             fn.argtypes = args
             fn.restype = _I
+        L.rb_plan_begin.argtypes, L.rb_plan_begin.restype = [], _P
+        L.rb_plan_end.argtypes, L.rb_plan_end.restype = [_P], _I
+        L.rb_plan_calls.argtypes, L.rb_plan_calls.restype = [_P], _I
+        L.rb_plan_replay.argtypes, L.rb_plan_replay.restype = [_P, _P], _I
+        L.rb_plan_free.argtypes, L.rb_plan_free.restype = [_P], None
         L.rb_gemm_workspace_floats.argtypes = [_I, _I, _I, _I]
         L.rb_gemm_workspace_floats.restype = ctypes.c_longlong
         L.rb_sample_workspace_bytes.argtypes = [_I, _I]
@@ -405,6 +410,28 @@ class Kernels:
             raise KernelError("sampling workspace too small")
         self._ok(self._lib.rb_sample(_ptr(logits), n, vocab, _ptr(temperature), _ptr(u), _ptr(tokens),
                                      _ptr(workspace), self._stream()))
+
+    # ------------------------------------------------------------------ recorded steps
+    def plan_begin(self) -> int:
+        """From here to `plan_end` every launch of this thread is noted as well as issued; returns
+        the plan's handle."""
+        plan = self._lib.rb_plan_begin()
+        if not plan:
+            raise KernelError(self._lib.rb_last_error().decode("utf-8", "replace"))
+        return plan
+
+    def plan_end(self, plan: int) -> int:
+        """Ends the recording; returns the number of launches the plan holds."""
+        self._ok(self._lib.rb_plan_end(plan))
+        return int(self._lib.rb_plan_calls(plan))
+
+    def plan_replay(self, plan: int) -> None:
+        """Issues the plan's launches again on torch's current stream, with the arguments they were
+        recorded with: the memory those name must still be the step's own."""
+        self._ok(self._lib.rb_plan_replay(plan, self._stream()))
+
+    def plan_free(self, plan: int) -> None:
+        self._lib.rb_plan_free(plan)
 
     # ------------------------------------------------------------------ load time
     def fill_normal(self, out: torch.Tensor, key: int, mean: float, std: float) -> None:

@@ -195,6 +195,7 @@ extern "C" int rb_sample_workspace_bytes(int n_rows, int vocab) {
 
 extern "C" int rb_sample(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,
                          int32_t* tokens, void* workspace, void* stream) {
+  RB_RECORDED(rb_sample(logits, n_rows, vocab, temperature, u, tokens, workspace, stream));
   RB_REQUIRE(n_rows >= 0 && vocab > 0, "rb_sample: bad sizes %d x %d", n_rows, vocab);
   RB_REQUIRE(temperature == nullptr || u != nullptr, "rb_sample: temperature given without uniform numbers");
   RB_REQUIRE(workspace != nullptr, "rb_sample: no workspace");

@@ -140,6 +140,7 @@ class StepContext:
         self.host_slots: List[int] = []
         self.host_past: List[int] = []
         self._workspaces: Dict[Tuple[int, int, int, int], Tuple] = {}
+        self._copied: Optional[torch.cuda.Event] = None      # the last copy of the host buffer to the device
 
     @classmethod
     def for_batch(cls, device, batch: StepBatch, n_compute_units: int) -> "StepContext":
@@ -151,6 +152,8 @@ class StepContext:
 
     def fill(self, batch: StepBatch) -> None:
         """Writes the batch into the layout and copies it to the GPU (one copy)."""
+        if self._copied is not None:
+            self._copied.synchronize()        # the copy before this one has read the host buffer
         q_lens = [len(t) for t in batch.tokens]
         b, t = len(batch.slots), int(sum(q_lens))
         if b != self.n_seqs or t != self.n_tokens or len(batch.rows) != self.n_rows:
@@ -186,6 +189,10 @@ class StepContext:
         if self.fixed_bucket is None:
             self.bucket = split_bucket(self.max_kv_len)
         self._dev.copy_(self._host, non_blocking=True)
+        if self._host.is_pinned():
+            if self._copied is None:
+                self._copied = torch.cuda.Event()
+            self._copied.record()
 
     def decode_workspace(self, n_heads: int, head_dim: int, n_kv_heads: int = 1) -> Tuple:
         """Split count and scratch for decode attention: enough workgroups to fill the

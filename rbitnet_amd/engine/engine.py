@@ -58,6 +58,11 @@ class Engine:
         self.use_graphs = bool(model.graph_safe) and getattr(self.lib, "times", None) is None
         # (rows of the captured step, split bucket) -> DecodeGraph, least recently used first
         self._graphs: "OrderedDict[Tuple[int, int], Any]" = OrderedDict()
+        # steps other than the captured decode step: launches issued from C++ once a shape has been seen
+        # before (step_plan.py); only for models whose parts do nothing on the device but call the library
+        self.use_plans = bool(getattr(model, "plan_safe", False)) and getattr(self.lib, "times", None) is None
+        from .step_plan import StepPlans
+        self.plans = StepPlans(self)
         # float32 [sequences, vocab] of the last `decode_step`, valid until the next one
         self.last_decode_logits: Optional[torch.Tensor] = None
         from ..sampling import Sampler
@@ -200,9 +205,11 @@ class Engine:
             base += len(toks)
         q_lens = [len(t) for t in tokens]
         self.cache.reserve(slots, q_lens)
-        ctx = StepContext.for_batch(self.device, StepBatch(slots, past, tokens, rows, self.cache.block_tables(slots)),
-                                    n_compute_units=self.lib.n_compute_units)
-        logits = self.model.forward(ctx, self.cache, ctx.rows)
+        batch = StepBatch(slots, past, tokens, rows, self.cache.block_tables(slots))
+        logits = self.plans.run(batch) if self.use_plans else None
+        if logits is None:
+            ctx = StepContext.for_batch(self.device, batch, n_compute_units=self.lib.n_compute_units)
+            logits = self.model.forward(ctx, self.cache, ctx.rows)
         self.cache.commit(slots, q_lens)
         self.stats["steps"] += 1
         if max(q_lens) == 1:

@@ -119,6 +119,12 @@ class Model:
     def graph_safe(self) -> bool:
         return all(getattr(p, "graph_safe", False) for p in list(self.blocks) + [self.embedding, self.head])
 
+    @property
+    def plan_safe(self) -> bool:
+        """Whether every part's forward does nothing on the device but call the kernel library, so
+        that a step's launches can be recorded there and issued again from C++."""
+        return all(getattr(p, "plan_safe", False) for p in list(self.blocks) + [self.embedding, self.head])
+
     def max_positions(self) -> int:
         return self.spec.max_positions
 

@@ -41,6 +41,7 @@ _DECODE_GROUPS = tuple(range(1, 17))    # query heads per kv head the decode ker
 
 class Attention(Part):
     graph_safe = True
+    plan_safe = True
     takes_gained_rows = True
     adds_to_stream = True
 
@@ -60,6 +61,7 @@ class Attention(Part):
         self.cache_from = params.get("cache_from")
         self.names = dict(DEFAULT_NAMES, **(params.get("names") or {}))
         self.position = build_part("position", params["position"], env)
+        self.plan_safe = bool(getattr(self.position, "plan_safe", False))
         self.hidden = env.hidden_size
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_q: Optional[torch.Tensor] = None

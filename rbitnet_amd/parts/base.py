@@ -83,6 +83,10 @@ class Part:
     # synchronisation, no host-side reads of device data): the decode step may then be
     # captured into a HIP graph.  A part that does not say so is run launch by launch.
     graph_safe = False
+    # True when forward does nothing on the device but call the kernel library (no torch operation of
+    # its own that computes or copies): the launches of a step can then be recorded in the library and
+    # issued again from C++ for the next step of the same shape.
+    plan_safe = False
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {}

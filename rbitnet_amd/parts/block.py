@@ -43,6 +43,10 @@ class PreNormBlock:
     def graph_safe(self) -> bool:
         return all(getattr(p, "graph_safe", False) for p in (self.norm1, self.mixer, self.norm2, self.feed_forward))
 
+    @property
+    def plan_safe(self) -> bool:
+        return all(getattr(p, "plan_safe", False) for p in (self.norm1, self.mixer, self.norm2, self.feed_forward))
+
     def parts(self) -> Dict[str, object]:
         return {self.segments["norm1"]: self.norm1, self.segments["mixer"]: self.mixer,
                 self.segments["norm2"]: self.norm2, self.segments["feed_forward"]: self.feed_forward}

@@ -35,6 +35,7 @@ from .stream import normed_for
 
 class TableEmbedding(Part):
     graph_safe = True
+    plan_safe = True
 
     def __init__(self, params: Dict, env: BuildEnv):
         self.env = env
@@ -73,6 +74,10 @@ class LinearHead(Part):
     @property
     def graph_safe(self) -> bool:
         return bool(getattr(self.norm, "graph_safe", False))
+
+    @property
+    def plan_safe(self) -> bool:
+        return bool(getattr(self.norm, "plan_safe", False))
 
     @property
     def first_norm(self):

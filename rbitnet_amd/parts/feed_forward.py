@@ -25,6 +25,7 @@ DEFAULT_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "do
 
 class SwiGLU(Part):
     graph_safe = True
+    plan_safe = True
     takes_gained_rows = True
     adds_to_stream = True
 

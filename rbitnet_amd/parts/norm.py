@@ -29,6 +29,7 @@ from .stream import GainedRows  # noqa: F401  (its old home; importers find it h
 
 class RMSNorm(Part):
     graph_safe = True
+    plan_safe = True
     folds_into_products = True
     adds_terms = True
 

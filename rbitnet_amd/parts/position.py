@@ -55,6 +55,7 @@ def rope_inverse_frequencies(head_dim: int, theta: float, scaling: Optional[Dict
 
 class Rope(Part):
     graph_safe = True
+    plan_safe = True
     takes_terms = True      # qkv may come as [P, T, W]: terms that the kernel adds up
 
     def __init__(self, params: Dict, env: BuildEnv):
@@ -92,6 +93,7 @@ class Rope(Part):
 
 class NoPosition(Part):
     graph_safe = True
+    plan_safe = True
     takes_terms = True
 
     def __init__(self, params: Dict, env: BuildEnv):
