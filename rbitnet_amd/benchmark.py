@@ -157,6 +157,32 @@ def generate_run(engine, n_requests: int, prompt_len: int, seed: int = 0, lo: in
     return out
 
 
+def short_prompts_run(engine, lengths, runs: int = 7) -> dict:
+    """One prompt of each length, `runs` times: the step's wall time launched from Python and issued
+    from C++ as a recorded step (the median of the runs after the one that records)."""
+    import numpy as np
+    rng = np.random.default_rng(5)
+    out = {}
+    for n in lengths:
+        prompt = [int(t) for t in rng.integers(0, engine.spec.vocab_size, size=n)]
+        row = {}
+        for label, plans in (("python_ms", False), ("recorded_ms", True)):
+            engine.use_plans = plans
+            times = []
+            for _ in range(runs + 2):
+                slot = engine.alloc_slot()
+                _sync()
+                t0 = time.perf_counter()
+                engine.step([(slot, prompt)], "last")
+                _sync()
+                times.append(time.perf_counter() - t0)
+                engine.free_slot(slot)
+            row[label] = round(sorted(times[2:])[runs // 2] * 1e3, 3)
+        out[str(n)] = row
+    engine.use_plans = True
+    return out
+
+
 def probe(lib, device) -> dict:
     """What this GPU reaches on a streaming read (`read_*`: all workgroups striding through the
     buffer together with plain loads; `stream_*`: every workgroup walking pieces of its own with
@@ -216,6 +242,9 @@ def main(argv=None) -> int:
     ap.add_argument("--generate", type=int, default=0, metavar="N",
                     help="no benchmark line: Engine.generate for N requests with limits drawn from 16..256 against "
                          "captured steps of fixed batches (see generate_run)")
+    ap.add_argument("--short-prompts", default="", metavar="N,N,...",
+                    help="no benchmark line: one prompt of each of these lengths, launched from Python and issued "
+                         "from C++ as a recorded step")
     ap.add_argument("--tokens", default="1,8,64,512,2048", help="token counts of --planner-sweep")
     ap.add_argument("--sweep-detail", default=None, help="--planner-sweep: a file for every candidate's time")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
@@ -267,6 +296,9 @@ def main(argv=None) -> int:
     _sync()
     if args.generate:
         print(json.dumps(generate_run(engine, args.generate, longest)))
+        return 0
+    if args.short_prompts:
+        print(json.dumps(short_prompts_run(engine, [int(v) for v in args.short_prompts.split(",") if v])))
         return 0
 
     dt, ctx_mean = decode_run(engine, args.batch, args.steps, args.warmup, prompt_len=prompt_len)

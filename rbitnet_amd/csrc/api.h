@@ -130,6 +130,9 @@ int rb_sample(const float* logits, int n_rows, int vocab, const float* temperatu
 // 128k vocabulary); more is refused with an error and nothing is launched.  The stream must belong
 // to the current device.  All calls on one GPU share that memory: two calls whose kernels may
 // overlap there (different streams, no dependency between them) race; calls on one stream do not.
+// The first use on a device asks the runtime for the address of that device's copy; before the
+// first call under stream capture, call rb_sample_static_max_stats() (or rb_sample_static once) on
+// that device outside of any capture.
 int rb_sample_static_max_stats(void);
 int rb_sample_static(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,
                      int32_t* tokens, void* stream);

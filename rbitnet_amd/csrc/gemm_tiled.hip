@@ -589,17 +589,15 @@ static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, in
 }
 
 // ------------------------------------------------------------------ which tiles, how many K slices
-// Measured on the Llama-3-8B products (N = 4096 .. 28672, K = 4096 and 14336) from 17 to 8,192
-// tokens.  The kernels are bound by what they pull from L2 and LDS (a 128 x 128 x 64 tile needs
-// a byte per 64 flop, a 256 x 256 one half of that), so the largest tile that still gives
-// every compute unit work wins, and where even the smallest tiles are too few, K is cut into
-// slices over workgroups (grid.y): each slice writes its partial sums to its own [M, N] slab
-// of a workspace, and gemm_sum_slabs_kernel adds them up in a fixed order.
-//   cfg 4: 256 x 256 (8 waves)        at least ~160 such tiles
-//   cfg 6: 192 x 256 (8 waves)        ... when that fills the last round of workgroups better
-//   cfg 5: 128 x 128 (4 waves, 2 workgroups per compute unit)
-//   cfg 7: 128 rows of W x 64 tokens, 3 stages deep    up to 512 tokens, when cfg 5 has < 256 tiles
-//   cfg 10, 13: its variants for wide gated products of at most 64 tokens (see plan_tiles)
+// The kernels are bound by what they pull from L2 and LDS (a 128 x 128 x 64 tile needs a byte per
+// 64 flop, a 256 x 256 one half of that), so the largest tile that still gives every compute unit
+// work wins, and where even the smallest tiles are too few, K is cut into slices over workgroups
+// (grid.y): each slice writes its partial sums to its own [M, N] slab of a workspace, and
+// gemm_sum_slabs_kernel (or the kernel that reads them) adds them up in a fixed order.
+//   cfg 4: 256 rows of W x 256 tokens (8 waves)      cfg 6: 192 x 256      cfg 9: 320 x 256
+//   cfg 8: 256 x 128, 3 stages deep                  cfg 5: 128 x 128 (4 waves, 2 workgroups per compute unit)
+//   cfg 7: 128 x 64, 3 stages deep (2 per compute unit)      cfg 13: the same with K tiles of 128
+//   cfg 10: 64 x 64, 4 stages deep (2 per compute unit)
 //   cfg 1..3: tiles staged through registers, for K that is no multiple of 64 (more than 64 tokens)
 // Without K slices a product of 128 tokens by 4096 rows ran on 32 of the 256 compute units and
 // took as long as one of 768 tokens (K = 14336: 194 us; 41 us with 4 slices of 64-token tiles).
@@ -614,27 +612,72 @@ extern "C" void rb_tune_tiles(int cfg, int parts) {       // experiments only; 0
   g_tile_parts = parts;
 }
 
-// The most slices that keep the workgroups within `slots`, the slices at least 4 tiles deep
-// and equal, and their number within `cap` (every slice writes and re-reads an [M, N] slab,
-// 8 bytes per element, against W's 2 N K bytes).
-static int k_slices(long long tiles, int k, long long slots, int cap) {
+// The choice among the direct-to-LDS tiles and the number of K slices is the least of an estimate
+// of every candidate's time, a sum whose terms were fitted to 4,146 measured products (the four
+// products of a layer of six model shapes, hidden sizes 2,048 to 8,192, at 32 to 4,096 tokens,
+// every tile with 1 to 8 slices forced in turn; `bench.py --planner-sweep` repeats the sweep):
+//
+//   time [us] = c0 + tiles on the busiest compute unit x (K tiles of a slice x a + b)
+//               + slab x (MB of partial sums, when K is cut) + gate x (millions of gated outputs)
+//
+// A launch of w workgroups puts ceil(w / compute units) of them on the busiest compute unit; of a tile
+// that fits twice on one (128 x 128, 128 x 64, 64 x 64) two run side by side, and a pair costs `pair`
+// per K tile in place of 2 a.  The machine enters through the number of compute units alone.  The
+// estimate's own choice is within 5 % of the best candidate in 123 of the 132 products of more than
+// 64 tokens (mean 0.8 % above the best, 14.7 % at worst) and in 41 of the 48 of 17 to 64 tokens
+// (1.2 %, 7.3 %); fitted to three of the shapes it does as well on the other three.
+struct TileCost {
+  int cfg, rows, tokens, bk;
+  float a, b, pair;        // pair 0: one workgroup to a compute unit
+};
+struct CostTable {
+  float c0, slab, gate;
+  const TileCost* tiles;
+  int n_tiles;
+};
+static const TileCost kCostMany[] = {
+    {4, 256, 256, 64, 1.3576f, 2.676f, 0.f},    {5, 128, 128, 64, 0.8132f, 0.224f, 1.0457f},
+    {6, 192, 256, 64, 1.2159f, 1.570f, 0.f},    {7, 128, 64, 64, 0.4139f, 0.223f, 0.7074f},
+    {8, 256, 128, 64, 0.8527f, 1.438f, 0.f},    {9, 320, 256, 64, 1.5111f, 5.236f, 0.f},
+    {10, 64, 64, 64, 0.2674f, 0.252f, 0.4422f}, {13, 128, 64, 128, 0.4171f, 1.6625f, 0.f}};
+static const TileCost kCostFew[] = {{7, 128, 64, 64, 0.4221f, -1.565f, 1.0042f},
+                                    {10, 64, 64, 64, 0.2536f, -1.024f, 0.5691f},
+                                    {13, 128, 64, 128, 0.4052f, -0.410f, 0.f}};
+static const CostTable kMany = {3.744f, 0.4532f, 0.7218f, kCostMany, 8};      // more than 64 tokens
+static const CostTable kFew = {5.742f, 1.0625f, 3.6146f, kCostFew, 3};        // 17 to 64 tokens
+
+static TilePlan plan_by_cost(int m, int n, int k, int epilogue) {
+  const CostTable& table = m > 64 ? kMany : kFew;
+  const long long cus = rb_compute_units();
   const int kt = k / 64;
-  if (cap > 16) cap = 16;
-  int best = 1;
-  for (int p = 1; p <= cap; ++p)
-    if (kt % p == 0 && kt / p >= 4 && tiles * p <= slots) best = p;
+  TilePlan best = {0, 1};
+  double best_cost = 0.0;
+  for (int i = 0; i < table.n_tiles; ++i) {
+    const TileCost& t = table.tiles[i];
+    if (k % t.bk != 0) continue;
+    const long long tiles = (long long)((n + t.rows - 1) / t.rows) * ((m + t.tokens - 1) / t.tokens);
+    for (int p = 1; p <= (epilogue ? 1 : 8); ++p) {
+      if ((k / t.bk) % p != 0 || (p > 1 && kt / p < 4)) continue;
+      const long long busiest = (tiles * p + cus - 1) / cus;
+      const double per_k = t.pair > 0.f ? (busiest % 2) * t.a + (busiest / 2) * t.pair : busiest * t.a;
+      double cost = table.c0 + (double)kt / p * per_k + busiest * t.b;
+      if (p > 1) cost += table.slab * (4e-6 * p * m * n);
+      if (epilogue) cost += table.gate * (1e-6 * m * n);
+      if (best.cfg == 0 || cost < best_cost) {
+        best = {t.cfg, p};
+        best_cost = cost;
+      }
+    }
+  }
   return best;
 }
 
 static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
-  // One round: a workgroup on every compute unit.  The thresholds below are the measured ones of a GPU
-  // with 256 compute units, kept as fractions of a round (5/8, 11/16, 3/4, 25/32, 7/8, 1, 3/2, 2).
   const long long R = rb_compute_units();
-  const auto rounds = [R](long long tiles) { return (tiles + R - 1) / R; };
   const bool dma = k % 64 == 0 && (long long)k * 512 < (1LL << 32);
-  const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
   if (!dma) {
     if (m <= 64) return {0, 1};
+    const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
     const long long t256x128 = (long long)((m + 127) / 128) * ((n + 255) / 256);
     if (g_tile_cfg >= 1 && g_tile_cfg <= 3) return {g_tile_cfg, 1};
     return {t256 >= R * 5 / 8 ? 3 : (k >= 8192 && t256x128 >= R * 25 / 32 ? 2 : 1), 1};
@@ -644,121 +687,7 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
     const int p = (epilogue == 0 && g_tile_parts > 0 && (k / 64) % g_tile_parts == 0) ? g_tile_parts : 1;
     return {g_tile_cfg, p};
   }
-  const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
-  const long long t64 = (long long)((m + 63) / 64) * ((n + 127) / 128);
-  // Rows that divide into 320-row tiles exactly, in a deep product: those tiles in 2 or 4 K slices where that
-  // makes one round (10,240 rows at K = 8192: 512 tokens 77 us in 4 slices against 100 in 2 slices of
-  // 256 x 128 tiles, 1,024 tokens 135 in 2 slices against 180 in one round of 216 tiles of 192 rows).
-  // Only with tiles of tokens that are nearly full and a round that is nearly full (768 tokens, 192
-  // workgroups: slower than one round of the 256 x 128 tiles).
-  if (m > 64 && epilogue == 0 && n % 320 == 0 && (m + 255) / 256 * 256 - m <= m / 8) {
-    const long long t320x = (long long)((m + 255) / 256) * (n / 320);
-    for (int p = 2; p <= 4; p *= 2)
-      if (t320x * p >= R * 7 / 8 && t320x * p <= R && (k / 64) % p == 0 && k / 64 / p >= 32) return {9, p};
-  }
-  if (m > 64 && t256 >= R * 5 / 8) {
-    // rounds of 256 workgroups times the time of a tile: a 192-row tile does 0.75 of the work
-    // of a 256-row one in 0.81 of the time, a 320-row tile 1.25 of it in 1.22 to 1.26 (28,672 gated
-    // rows by 2,048 tokens: 896 tiles of 256 rows, 3.5 rounds, 475 us; 720 of 320 rows, under 3
-    // rounds, 459 us).  Checked against the fastest of the three for 28,672 gated rows at 384 to
-    // 4,096 tokens in steps of 128, and for 6,144 and 4,096 rows: within 2 % everywhere.
-    const long long t192 = (long long)((m + 255) / 256) * ((n + 191) / 192);
-    const long long t320 = (long long)((m + 255) / 256) * ((n + 319) / 320);
-    const long long cost256 = rounds(t256) * 1000, cost192 = rounds(t192) * 815, cost320 = rounds(t320) * 1220;
-    // Tiles of 256 rows x 128 tokens, 0.65 of the time of 256 x 256, where the last tile of 256 tokens
-    // would be mostly empty (57,344 gated rows at K = 8192: 96 tokens 143 us against 224, 288 tokens 375
-    // against 414).
-    const long long t128t = (long long)((m + 127) / 128) * ((n + 255) / 256);
-    const long long cost128t = rounds(t128t) * 650;
-    // A very deep product in 2 K slices of the 256 x 256 tiles where that fills the last round better (8,192
-    // rows at K = 28672, 3,072 tokens: 384 tiles, one and a half rounds that take the time of two; 768 half
-    // tiles make three rounds of half the time: 1,125 us against 1,300, and 40 us for the second slab).
-    if (epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 128) {
-      const long long cost256x2 = rounds(2 * t256) * 500 + 60;
-      if (cost256x2 < cost256 && cost256x2 < cost192 && cost256x2 < cost320 && cost256x2 < cost128t) return {4, 2};
-    }
-    if (cost128t < cost256 && cost128t < cost192 && cost128t < cost320) return {8, 1};
-    if (cost320 < cost256 && cost320 < cost192) return {9, 1};
-    return {cost192 < cost256 ? 6 : 4, 1};
-  }
-  // 256 rows x 128 tokens, 3 stages deep, where such tiles fill one round of 256 workgroups (or
-  // three quarters of it): measured against the 128 x 128 tiles that would run two to a compute
-  // unit, 2,048 tokens by 4,096 rows 237 us against 258 at K = 14336 and 82.6 against 83.6 at
-  // K = 4096; 1,024 tokens by 6,144 rows 76 against 82; 256 tokens by 28,672 gated rows 80 against
-  // 89.  With fewer or more tiles than that they lose (1,024 tokens by 4,096 rows: 204 against 159).
-  // Where they are half, a quarter or an eighth of a round, K is cut into 2, 4 or 8 slices of at least 32,
-  // 16 and 24 tiles (256 tokens by 4,096 rows at K = 14336: 41 us in 8 slices against 59; at K = 4096 in
-  // 4 slices, 512 tokens by 4,096 rows 24 us against 30, 256 by 6,144 24 against 30; 128 by 12,288 28 against 33,
-  // but there the four slabs cost the kernel that adds them more than that),
-  // which fills the round again: 512 tokens by 4,096 rows at K = 14336 75 us in 4 slices against 107
-  // in the 64-token tiles (320 tokens: 64 against 106), 1,024 tokens 127 in 2 slices against 146 in
-  // 128 x 128 tiles; at K = 4096, 768 tokens by 4,096 rows 46 against 59, 512 by 6,144 48 against 56.
-  // 160 workgroups of 2 slices still win (640 tokens by 4,096 rows: 43 against 58), 144 do not.
-  const long long t256x128 = (long long)((m + 127) / 128) * ((n + 255) / 256);
-  // A deep product (K >= 8192) whose 256 x 256 tiles are half a round goes in 2 slices of those
-  // rather than in one round of the 256 x 128 tiles (4,096 rows at K = 14336: 2,048 tokens 197 us
-  // against 220, 1,536 tokens 172 against 195; the second slab costs the norm that adds it about 10).
-  if (m > 64 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 64 && t256 * 2 >= R * 3 / 4 && t256 * 2 <= R)
-    return {4, 2};
-  // and where they are a quarter of a round, in 4 slices (768 tokens: 94 us against 106 in 2 slices of the
-  // 256 x 128 tiles; 1,024 tokens: 109 against 118)
-  if (m > 64 && epilogue == 0 && (k / 64) % 4 == 0 && k / 64 / 4 >= 48 && t256 * 4 >= R * 3 / 4 && t256 * 4 <= R)
-    return {4, 4};
-  // an eighth of a round, of a very deep product, in 8 (8,192 rows at K = 28672, 256 tokens: 122 us against 141
-  // in 4 slices of the 256 x 128 tiles)
-  if (m > 128 && epilogue == 0 && (k / 64) % 8 == 0 && k / 64 / 8 >= 48 && t256 * 8 >= R * 3 / 4 && t256 * 8 <= R)
-    return {4, 8};
-  // (a gated product, whose K cannot be cut, from 160 such tiles on: 22,016 gated rows, 256 tokens, 172
-  // tiles 64 us against 74 in 344 tiles of 128 x 128)
-  if (m > 64 && t256x128 >= (epilogue == 1 ? R * 5 / 8 : R * 3 / 4) && t256x128 <= R) return {8, 1};
-  if (m > 64 && epilogue == 0) {
-    for (int p = 2; p <= 8; p *= 2)
-      if (t256x128 * p >= R * 5 / 8 && t256x128 * p <= R && (k / 64) % p == 0 && k / 64 / p >= (p == 2 ? 32 : (p == 4 ? (n <= 8192 ? 16 : 32) : 24)))
-        return {8, p};
-  }
-  // Between one and two thousand tokens the large tiles are too few for a round by themselves: a deep
-  // product (K >= 8192) is cut into 2 slices of them (1,152 tokens by 4,096 rows at K = 14336: 164 us in
-  // 192 x 256 tiles against 204 in 128 x 128; 1,408 tokens: 182 in 256 x 256 against 208), and where
-  // 192 x 256 tiles alone make most of a round they are taken (1,408 tokens by 6,144 rows: 86 against 110).
-  const long long t192r = (long long)((m + 255) / 256) * ((n + 191) / 192);
-  if (m > 64 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 64) {
-    if (t192r * 2 >= R * 5 / 8 && t192r * 2 <= R) return {6, 2};
-    if (t256 * 2 >= R * 5 / 8 && t256 * 2 <= R) return {4, 2};
-  }
-  // (at K = 4096 where the 192-row tiles in 2 slices make three quarters of a round or more, up to 768
-  // tokens, beyond which the second slab costs more than that: 12,288 rows, 384 tokens 51 us against 65;
-  // 6,144 rows, 768 tokens 50 against 60)
-  if (m > 64 && m <= 768 && epilogue == 0 && (k / 64) % 2 == 0 && k / 64 / 2 >= 32 && t192r * 2 >= R * 3 / 4 && t192r * 2 <= R)
-    return {6, 2};
-  if (m > 64 && t192r >= R * 11 / 16 && t192r <= R) return {6, 1};
-  if (m > 64 && (t128 >= R || m > 512)) return {5, epilogue ? 1 : k_slices(t128, k, 2 * R, k / (4 * m))};
-  // A gated product of at most 64 tokens cannot cut K and streams W from too few workgroups to
-  // hide anything (28,672 rows: 224 tiles of 128): tiles of 64 rows, four stages deep, two to a
-  // compute unit, up to 24 tokens (17 tokens: 45 us against 50), and K tiles of 128 (256 bytes a
-  // row and load) beyond (64 tokens: 49.2 against 50.8).
-  // The 64-row tiles only where they are at least one and a half to a compute unit (22,016 gated rows, 344
-  // tiles, 17 tokens: 37 us against 34 with K tiles of 128), and with a deep K the plain 128 x 64 tiles
-  // (57,344 gated rows at K = 8192: 139-147 us against 146-155 at 17 to 64 tokens).
-  if (m <= 64 && epilogue == 1 && n >= 16384 && k < 8192) {
-    if (m <= 24 && (n + 63) / 64 >= R * 3 / 2) return {10, 1};
-    if (k % 128 == 0) return {13, 1};
-  }
-  // At most 64 tokens, no gate: tiles of 128 rows in K slices, or tiles of 64 rows (four stages deep, two
-  // to a compute unit) in half as many slices.  The small tiles where they make more workgroups, up to
-  // one per compute unit (4,096 rows at K = 11008, whose 172 K tiles go in 4 slices and not in 8: 19.5 us
-  // in 256 workgroups against 26.6 in 128), and at equal numbers where K is short (K = 4096: 4,096 rows
-  // 9.8 us in 4 slices against 11.1-12.9 in 8, 6,144 rows 13.4 against 14.2; K = 8192: 8,192 rows 24.9
-  // against 26.0): the kernel that adds the slabs then has half as many to add.  With a long K the
-  // large tiles win at equal numbers (4,096 rows at K = 14336: 22.2 us against 23.3), and so they do
-  // against small tiles in one slice (10,240 rows at K = 8192: 35.3 against 40.2).
-  if (m <= 64 && epilogue == 0) {
-    const int pa = k_slices(t64, k, R, k / (8 * m));
-    const int pb = k_slices((n + 63) / 64, k, R, 8);
-    const long long wa = t64 * pa, wb = (long long)((n + 63) / 64) * pb;
-    if (wb <= R && (wb > wa || (wb == wa && pb >= 2 && k <= 8192))) return {10, pb};
-    return {7, pa};
-  }
-  return {7, epilogue ? 1 : k_slices(t64, k, R, k / (8 * m))};
+  return plan_by_cost(m, n, k, epilogue);
 }
 
 template <int EPI, typename TO, bool WF>

@@ -241,7 +241,14 @@ static int scratch_of_current_device(void** out) {
   return 0;
 }
 
-extern "C" int rb_sample_static_max_stats(void) { return SAMPLE_STATIC_MAX_STATS; }
+// Also the set-up call: it asks for the current device's copy of the scratch array, so that a first
+// rb_sample_static under stream capture finds the address known (the runtime may refuse the query
+// while a stream captures).
+extern "C" int rb_sample_static_max_stats(void) {
+  void* ptr = nullptr;
+  (void)scratch_of_current_device(&ptr);
+  return SAMPLE_STATIC_MAX_STATS;
+}
 
 extern "C" int rb_sample_static(const float* logits, int n_rows, int vocab, const float* temperature, const float* u,
                                 int32_t* tokens, void* stream) {

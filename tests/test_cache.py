@@ -140,3 +140,51 @@ def test_state_is_reset_when_a_slot_is_handed_out():
     st[s] += 5
     c.free_slot(s)
     assert c.alloc_slot() == s and torch.all(c.view(0, {}).state[s] == 2.0)
+
+
+def test_a_third_kind_of_group_registered_from_here():
+    """A paged group of the test's own (one number per position and layer, shown to its mixer in a
+    field of its own) beside the built-in kinds: reserved, committed, grown, freed and checked like them."""
+    from rbitnet_amd.cache.cache import PagedGroup, register_cache_kind
+
+    class MarksGroup(PagedGroup):
+        kind = "marks"
+
+        def __init__(self, request, layers, n_pages, n_slots, dtype, device):
+            super().__init__(request, layers, n_pages)
+            self.marks = torch.zeros((len(self.layers), n_pages + 1, PAGE_SIZE), dtype=dtype, device=device)
+
+        @staticmethod
+        def bytes_per_token(request, n_layers, dtype):
+            return n_layers * torch.empty((), dtype=dtype).element_size()
+
+        def fill_view(self, view, i, block_tables):
+            view.marks = self.marks[i]
+            view.marks_table = block_tables[id(self)]
+
+        def bytes(self):
+            return self.marks.numel() * self.marks.element_size()
+
+    register_cache_kind("marks", MarksGroup)
+    reqs = [CacheRequest("kv", heads=1, head_dim=4), CacheRequest("marks"), CacheRequest("marks")]
+    c = Cache(reqs, 2, 64 * 3, torch.float32, "cpu")
+    marks = next(g for g in c.groups if g.kind == "marks")
+    assert marks in c.kv_groups and len(c.kv_groups) == 2 and marks.layers == [1, 2]
+    assert c.token_capacity() == 64 * 3
+    a, b = c.alloc_slot(), c.alloc_slot()
+    c.reserve([a, b], [100, 5])
+    c.commit([a, b], [100, 5])
+    tables = c.block_tables([a, b, c.spare_slot])
+    assert [len(t) for t in tables[id(marks)]] == [2, 1, 1] and tables[id(marks)][2] == [marks.spare_page]
+    view = c.view(2, {id(g): torch.tensor([[0]]) for g in c.kv_groups})
+    assert view.marks.shape == (3 + 1, PAGE_SIZE) and view.k_pages is None
+    assert not c.can_grow(a, 64) and c.can_grow(b, 59) and not c.can_grow(b, 60)       # both groups have one page left
+    with pytest.raises(CacheError, match="cache full"):
+        c.reserve([a, b], [29, 60])
+    c.check()
+    c.free_slot(a)
+    assert marks.table.pool.n_free == 2 and c.can_grow(b, 60)
+    c.free_slot(b)
+    c.check()
+    with pytest.raises(CacheError, match="keeps none"):           # only keys and values can be read by another layer
+        Cache([CacheRequest("marks"), None], 1, 64, torch.float32, "cpu", readers={1: 0})

@@ -46,13 +46,16 @@ def _both(lib, logits, temperature, u):
     rc = lib.rb_sample(logits.data_ptr(), rows, vocab, temperature.data_ptr(), u.data_ptr(), want.data_ptr(),
                        workspace.data_ptr(), stream)
     assert rc == 0, lib.rb_last_error()
+    assert lib.rb_sample_static_max_stats() > 0            # the set-up call: the scratch address is known from here on
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]             # the device's own count: an allocation past torch's would show
     rc = lib.rb_sample_static(logits.data_ptr(), rows, vocab, temperature.data_ptr(), u.data_ptr(), got.data_ptr(),
                               stream)
     assert rc == 0, lib.rb_last_error()
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     return got.cpu(), want.cpu()
 
 
@@ -74,6 +77,37 @@ def test_static_sampling_equals_the_workspace_one_twice_in_a_row():
     # and the first again: the larger call after the smaller
     got, want = _both(lib, *first)
     assert got.tolist() == want.tolist()
+
+
+def test_static_sampling_under_stream_capture():
+    """Recorded into a graph (what the entry point is for) and replayed with other inputs in the same
+    buffers, eager work and synchronisations between the replays: every replay equals rb_sample."""
+    lib = _library()
+    assert lib.rb_sample_static_max_stats() > 0            # outside the capture: asks for the scratch address
+    rows, vocab = 5, 33000
+    logits, temperature, u = _case(rows, vocab, 3, greedy_rows=(0,))
+    got = torch.full((rows,), -2, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = lib.rb_sample_static(logits.data_ptr(), rows, vocab, temperature.data_ptr(), u.data_ptr(), got.data_ptr(),
+                                  torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.rb_last_error()
+    workspace = torch.empty(lib.rb_sample_workspace_bytes(rows, vocab) // 8 + 1, dtype=torch.int64, device="cuda")
+    for replay in range(4):
+        new_logits, new_t, new_u = _case(rows, vocab, 10 + replay, greedy_rows=(replay % rows,))
+        logits.copy_(new_logits)
+        temperature.copy_(new_t)
+        u.copy_(new_u)
+        got.fill_(-2)
+        graph.replay()
+        want = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
+        rc = lib.rb_sample(logits.data_ptr(), rows, vocab, temperature.data_ptr(), u.data_ptr(), want.data_ptr(),
+                           workspace.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, lib.rb_last_error()
+        torch.cuda.synchronize()
+        assert got.tolist() == want.tolist(), f"replay {replay}"
+        _ = (torch.ones(4096, device="cuda") * 3).sum().item()          # unrelated eager work between the replays
 
 
 def test_static_sampling_refuses_what_its_scratch_cannot_hold():
