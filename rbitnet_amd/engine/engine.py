@@ -29,6 +29,11 @@ from .model import Model
 DEFAULT_MAX_BATCH = 8
 MAX_DECODE_GRAPHS = 24
 CACHE_MEMORY_FRACTION = 0.9       # of the memory that is free after the weights, for a cache nobody sized
+# A step's activations: the float32 stream, the projections before and after rotation, the gated
+# product's input and output, partial sums of products cut along K.  About this many values of 4 bytes
+# per token for every row of the widest matrix of a layer (measured at the 8B and 70B shapes: 3 to 4).
+ACTIVATION_ROWS_PER_TOKEN = 4
+STEP_TOKENS_SET_ASIDE = 8192      # a cache nobody sized leaves room for the activations of a step of this many tokens
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
            torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
@@ -93,6 +98,8 @@ class Engine:
         if per_token > 0 and model.device.type == "cuda":
             torch.cuda.empty_cache()          # what loading held for a moment counts as free
             free, _ = torch.cuda.mem_get_info(model.device)
+            if max_tokens is None:            # nobody sized the cache: a step's activations keep their room
+                free = max(0, free - model.activation_bytes(min(STEP_TOKENS_SET_ASIDE, max_batch * seq)))
             fits = int(free * CACHE_MEMORY_FRACTION) // per_token // PAGE_SIZE * PAGE_SIZE
         if max_tokens is not None:
             if pages_for(int(max_tokens)) * PAGE_SIZE > max(fits, PAGE_SIZE):
@@ -204,6 +211,15 @@ class Engine:
                 rows.append(base + int(j))
             base += len(toks)
         q_lens = [len(t) for t in tokens]
+        if sum(q_lens) > 1024 and self.device.type == "cuda":
+            # a long step's activations must fit beside the cache: say so before anything is reserved or launched
+            need = self.model.activation_bytes(sum(q_lens), len(rows))
+            free = torch.cuda.mem_get_info(self.device)[0] + torch.cuda.memory_reserved(self.device) \
+                - torch.cuda.memory_allocated(self.device)
+            if need > free:
+                raise InferenceError(
+                    f"a step of {sum(q_lens)} tokens needs about {need / 2**30:.1f} GiB for its activations and "
+                    f"{free / 2**30:.1f} GiB are free: feed the prompts in pieces, or make the cache smaller")
         self.cache.reserve(slots, q_lens)
         batch = StepBatch(slots, past, tokens, rows, self.cache.block_tables(slots))
         logits = self.plans.run(batch) if self.use_plans else None

@@ -168,6 +168,17 @@ class Model:
             total += own(esize) if own else _tensor_bytes(part.tensor_specs().values(), esize)
         return total
 
+    def activation_bytes(self, n_tokens: int, n_rows: int = 1) -> int:
+        """About what a step of n_tokens tokens that asks for n_rows rows of logits allocates beside
+        the weights and the cache (an estimate for sizing and for refusing a step early, not a bound)."""
+        from ..engine.engine import ACTIVATION_ROWS_PER_TOKEN
+        widest = self.spec.hidden_size
+        for prefix, part in _named_parts(self.spec, self.blocks).items():
+            for ts in part.tensor_specs().values():
+                if ts.role == "matrix" and len(ts.shape) == 2:
+                    widest = max(widest, int(ts.shape[0]))
+        return 4 * (ACTIVATION_ROWS_PER_TOKEN * widest * int(n_tokens) + 2 * self.spec.vocab_size * int(n_rows))
+
     # ------------------------------------------------------------------ forward
     def forward(self, ctx, cache, rows: torch.Tensor) -> torch.Tensor:
         """ctx.token_ids [T] -> float32 logits [len(rows), V] at the packed rows `rows`."""
