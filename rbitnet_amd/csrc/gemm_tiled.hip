@@ -613,22 +613,26 @@ extern "C" void rb_tune_tiles(int cfg, int parts) {       // experiments only; 0
 }
 
 // The choice among the direct-to-LDS tiles and the number of K slices is the least of an estimate
-// of every candidate's time, a sum whose terms were fitted to 4,146 measured products (the four
-// products of a layer of six model shapes, hidden sizes 2,048 to 8,192, at 32 to 4,096 tokens,
-// every tile with 1 to 8 slices forced in turn; `bench.py --planner-sweep` repeats the sweep):
+// of every candidate's time, a sum whose terms were fitted to 8,300 measured products: the four
+// products of a layer of six model shapes (hidden sizes 2,048 to 8,192) at 24 to 4,096 tokens, every
+// tile with 1 to 8 slices forced in turn (`bench.py --planner-sweep` repeats the sweep).
 //
-//   time [us] = c0 + tiles on the busiest compute unit x (K tiles of a slice x a + b)
+//   time [us] = c0 + K tiles of a slice x (what the compute units' tiles cost per K tile)
+//               + fixed x (tiles on the busiest compute unit)
 //               + slab x (MB of partial sums, when K is cut) + gate x (millions of gated outputs)
 //
-// A launch of w workgroups puts ceil(w / compute units) of them on the busiest compute unit; of a tile
-// that fits twice on one (128 x 128, 128 x 64, 64 x 64) two run side by side, and a pair costs `pair`
-// per K tile in place of 2 a.  The machine enters through the number of compute units alone.  The
-// estimate's own choice is within 5 % of the best candidate in 123 of the 132 products of more than
-// 64 tokens (mean 0.8 % above the best, 14.7 % at worst) and in 41 of the 48 of 17 to 64 tokens
-// (1.2 %, 7.3 %); fitted to three of the shapes it does as well on the other three.
+// A launch of w workgroups fills `slots` places at a time (the compute units, or twice as many for
+// the tiles of which two fit on one): w / slots full rounds at `full` each, and a last round of
+// rem workgroups.  A last round is cheaper than a full one and the cheaper the emptier (the
+// compute units that have work share the memory system with fewer): `last + per_fill x rem / units`,
+// and for the tiles that fit twice, once every unit has one, `second + per_second x (rem - units) / units`.
+// The machine enters through the number of compute units alone.  The estimate's own choice is
+// within 5 % of the best candidate in 258 of the 276 products of more than 64 tokens (0.8 % above
+// the best in the mean, 21 % at worst) and in 90 of the 96 of 17 to 64 tokens (0.8 %, 10 %); fitted
+// to the token counts that are powers of two alone it does as well on the others.
 struct TileCost {
-  int cfg, rows, tokens, bk;
-  float a, b, pair;        // pair 0: one workgroup to a compute unit
+  int cfg, rows, tokens, bk, per_unit;
+  float full, last, per_fill, second, per_second, fixed;
 };
 struct CostTable {
   float c0, slab, gate;
@@ -636,19 +640,23 @@ struct CostTable {
   int n_tiles;
 };
 static const TileCost kCostMany[] = {
-    {4, 256, 256, 64, 1.3576f, 2.676f, 0.f},    {5, 128, 128, 64, 0.8132f, 0.224f, 1.0457f},
-    {6, 192, 256, 64, 1.2159f, 1.570f, 0.f},    {7, 128, 64, 64, 0.4139f, 0.223f, 0.7074f},
-    {8, 256, 128, 64, 0.8527f, 1.438f, 0.f},    {9, 320, 256, 64, 1.5111f, 5.236f, 0.f},
-    {10, 64, 64, 64, 0.2674f, 0.252f, 0.4422f}, {13, 128, 64, 128, 0.4171f, 1.6625f, 0.f}};
-static const TileCost kCostFew[] = {{7, 128, 64, 64, 0.4221f, -1.565f, 1.0042f},
-                                    {10, 64, 64, 64, 0.2536f, -1.024f, 0.5691f},
-                                    {13, 128, 64, 128, 0.4052f, -0.410f, 0.f}};
-static const CostTable kMany = {3.744f, 0.4532f, 0.7218f, kCostMany, 8};      // more than 64 tokens
-static const CostTable kFew = {5.742f, 1.0625f, 3.6146f, kCostFew, 3};        // 17 to 64 tokens
+    {4, 256, 256, 64, 1, 1.5794f, 1.1882f, 0.3369f, 0.f, 0.f, 4.5309f},
+    {5, 128, 128, 64, 2, 1.0266f, 0.6988f, 0.1646f, 0.8664f, 0.2135f, 1.1148f},
+    {6, 192, 256, 64, 1, 1.3217f, 1.0321f, 0.3024f, 0.f, 0.f, 3.2531f},
+    {7, 128, 64, 64, 2, 0.6848f, 0.3279f, 0.1067f, 0.5481f, 0.2758f, 0.5548f},
+    {8, 256, 128, 64, 1, 0.9282f, 0.7138f, 0.2021f, 0.f, 0.f, 2.674f},
+    {9, 320, 256, 64, 1, 1.8295f, 1.3649f, 0.3086f, 0.f, 0.f, 7.2878f},
+    {10, 64, 64, 64, 2, 0.4365f, 0.1927f, 0.0777f, 0.3422f, 0.1646f, 0.384f},
+    {13, 128, 64, 128, 1, 0.4118f, 0.3109f, 0.1058f, 0.f, 0.f, 1.9912f}};
+static const TileCost kCostFew[] = {{7, 128, 64, 64, 2, 1.2099f, 0.3352f, 0.2479f, 0.8967f, 0.3f, -0.4082f},
+                                    {10, 64, 64, 64, 2, 0.6268f, 0.191f, 0.1144f, 0.4995f, 0.1176f, -0.1f},
+                                    {13, 128, 64, 128, 1, 0.6506f, 0.3182f, 0.2568f, 0.f, 0.f, 0.2565f}};
+static const CostTable kMany = {4.469f, 0.3738f, 0.2871f, kCostMany, 8};      // more than 64 tokens
+static const CostTable kFew = {5.522f, 0.6852f, 0.f, kCostFew, 3};            // 17 to 64 tokens
 
 static TilePlan plan_by_cost(int m, int n, int k, int epilogue) {
   const CostTable& table = m > 64 ? kMany : kFew;
-  const long long cus = rb_compute_units();
+  const long long units = rb_compute_units();
   const int kt = k / 64;
   TilePlan best = {0, 1};
   double best_cost = 0.0;
@@ -658,9 +666,12 @@ static TilePlan plan_by_cost(int m, int n, int k, int epilogue) {
     const long long tiles = (long long)((n + t.rows - 1) / t.rows) * ((m + t.tokens - 1) / t.tokens);
     for (int p = 1; p <= (epilogue ? 1 : 8); ++p) {
       if ((k / t.bk) % p != 0 || (p > 1 && kt / p < 4)) continue;
-      const long long busiest = (tiles * p + cus - 1) / cus;
-      const double per_k = t.pair > 0.f ? (busiest % 2) * t.a + (busiest / 2) * t.pair : busiest * t.a;
-      double cost = table.c0 + (double)kt / p * per_k + busiest * t.b;
+      const long long w = tiles * p, slots = units * t.per_unit;
+      const long long rounds = w / slots, rem = w - rounds * slots;
+      double per_k = rounds * t.full;
+      if (rem > 0 && rem <= units) per_k += t.last + t.per_fill * ((double)rem / units);
+      if (rem > units) per_k += t.second + t.per_second * ((double)(rem - units) / units);
+      double cost = table.c0 + (double)kt / p * per_k + t.fixed * ((w + units - 1) / units);
       if (p > 1) cost += table.slab * (4e-6 * p * m * n);
       if (epilogue) cost += table.gate * (1e-6 * m * n);
       if (best.cfg == 0 || cost < best_cost) {

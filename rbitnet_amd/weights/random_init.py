@@ -170,7 +170,7 @@ def write_random_model(folder: str, config: Any, seed: int = DEFAULT_SEED, std: 
     """config (dict, or path of a config.json) + seed -> folder with config.json
     and model.safetensors.  Returns the folder.  device: where the numbers are drawn (the
     same numbers everywhere; the GPU is far faster for large models); None: the GPU if there
-    is one."""
+    is one and the kernel library can be loaded, else the host."""
     from ..config import load_config
     from ..engine.model import expected_tensors
 
@@ -188,7 +188,14 @@ def write_random_model(folder: str, config: Any, seed: int = DEFAULT_SEED, std: 
         json.dump(raw, f, indent=2)
     layout = {n: (dtype, tuple(s.shape)) for n, s in expected.items()}
     if device is None:
-        device = "cuda:0" if torch.cuda.is_available() else "cpu"
+        device = "cpu"
+        if torch.cuda.is_available():
+            try:                          # the GPU when its kernels can be had, else the host twin: the same numbers
+                from ..csrc.lib import kernels
+                kernels()
+                device = "cuda:0"
+            except Exception:
+                pass
     save_file(os.path.join(folder, "model.safetensors"),
               ((n, t.cpu()) for n, t in random_tensors(expected, seed, std, norm_std, dtype, device)),
               metadata={"format": "pt", "seed": str(seed), "init_std": str(std), "norm_std": str(norm_std)},

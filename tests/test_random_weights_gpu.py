@@ -87,7 +87,7 @@ def test_a_seed_means_one_model_in_memory_and_on_disk(name, dtype, tmp_path):
     cfg, seed, norm_std = CONFIGS[name]
     store = torch.bfloat16 if dtype == "bfloat16" else torch.float32
     folder = rbitnet_amd.write_random_model(str(tmp_path / "m"), cfg, seed=seed, std=0.1, norm_std=norm_std,
-                                            dtype=store)
+                                            dtype=store, device="cpu")
     on_disk = rbitnet_amd.Engine.load_path(folder, dtype=dtype, max_tokens=256)
     in_memory = rbitnet_amd.Engine.random(cfg, seed=seed, dtype=dtype, std=0.1, norm_std=norm_std, max_tokens=256)
     other = rbitnet_amd.Engine.random(cfg, seed=seed + 1, dtype=dtype, std=0.1, norm_std=norm_std, max_tokens=256)
