@@ -10,7 +10,11 @@
 #include "gemm_internal.h"
 
 static int g_use_resident = 1, g_use_tiled_small = 1;
-extern "C" void rb_tune_use_resident(int on) { g_use_resident = on; }      // experiments only
+void gemm_resident_forced(int on);
+extern "C" void rb_tune_use_resident(int on) {      // experiments only
+  g_use_resident = on;
+  gemm_resident_forced(on == 2);
+}
 extern "C" void rb_tune_use_stream(int on) { g_use_tiled_small = on; }     // experiments only: 0 = skinny up to 64 tokens
 
 static int tiled_parts(int m, int n, int k, int epilogue) {

@@ -624,8 +624,9 @@ __global__ __launch_bounds__(512) void gemm_resident_kernel(const bf16_t* __rest
   }
 }
 
-static int g_res_tiles = 0;
+static int g_res_tiles = 0, g_res_forced = 0;
 extern "C" void rb_tune_resident(int tiles) { g_res_tiles = tiles; }      // experiments only; 0 = built-in
+void gemm_resident_forced(int on) { g_res_forced = on; }                  // set by rb_tune_use_resident(2)
 
 template <int MB, int XQ, int EPI, typename TO, bool SCALED>
 static int launch_resident(const GemmTokens& x, const bf16_t* w, void* c, const GemmAfter& after, int m, int n, int k,
@@ -660,6 +661,11 @@ static bool try_resident(const GemmTokens& x, const bf16_t* w, void* c, const Ge
   if (parts < 1 || slices % parts != 0) return false;
   const int n_waves = slices / parts;
   if (n_waves > 8) return false;
+  // With fewer than 7 waves a workgroup has too few loads in flight for the one compute unit it has to
+  // itself, and the skinny kernel, several workgroups to a compute unit, is faster (32,768 gated rows at
+  // K = 2048: 12.4 us against 13.8 with 4 waves; at K = 3072: 17.3 against 18.4 with 6); forced on
+  // (rb_tune_use_resident(2)) it still takes them.
+  if (n_waves < 7 && g_res_forced == 0) return false;
   if (EPI == 1 && (n % 32 != 0)) return false;
   if (FOLDS && (mb != 1 || parts != 1)) return false;
   if (mb == 1) {

@@ -19,6 +19,7 @@ idle rows: every kernel of a step computes a row from that row's inputs alone.
 """
 from __future__ import annotations
 
+import weakref
 from typing import Optional
 
 import torch
@@ -44,7 +45,7 @@ class DecodeGraph:
     again before every replay."""
 
     def __init__(self, engine, n_seqs: int, bucket: int = 16):
-        self.engine = engine
+        self.engine = weakref.proxy(engine)      # no cycle of references: the graphs go when the engine goes
         self.n_seqs = n_seqs
         # page tables as wide as a sequence of this graph can need: no longer than the engine
         # allows, than the cache has pages, or than the contexts of this split bucket reach

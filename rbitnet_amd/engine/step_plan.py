@@ -21,6 +21,8 @@ serves every other step: prompts, prompts in pieces, steps of a replayed trace.
 """
 from __future__ import annotations
 
+import gc
+import weakref
 from collections import OrderedDict
 from typing import Dict, Optional, Tuple
 
@@ -43,7 +45,9 @@ def plan_key(batch: StepBatch) -> Tuple:
 class StepPlan:
     def __init__(self, engine, key: Tuple):
         n_seqs, n_tokens, n_rows, _, widths, bucket = key
-        self.engine = engine
+        # no cycle of references with the engine: a plan and its pool go when the engine goes, at once,
+        # and not whenever the collector of cycles comes by
+        self.engine = engine if isinstance(engine, weakref.ProxyType) else weakref.proxy(engine)
         self.ctx = StepContext(engine.device, n_seqs, n_tokens, n_rows, dict(widths), bucket=bucket,
                                n_compute_units=engine.lib.n_compute_units)
         self.pool = torch.cuda.MemPool()
@@ -56,6 +60,10 @@ class StepPlan:
         eng = self.engine
         self.ctx.fill(batch)
         self.handle = eng.lib.plan_begin()
+        # While allocations go to this plan's pool no other pool may be destroyed (the allocator aborts):
+        # the collector of cycles, which might find an old engine's plans, waits until the step is recorded.
+        collecting = gc.isenabled()
+        gc.disable()
         try:
             with torch.cuda.use_mem_pool(self.pool, device=eng.device):
                 self.logits = eng.model.forward(self.ctx, eng.cache, self.ctx.rows)
@@ -63,6 +71,9 @@ class StepPlan:
             eng.lib.plan_free(self.handle)
             self.handle = None
             raise
+        finally:
+            if collecting:
+                gc.enable()
         self.calls = eng.lib.plan_end(self.handle)
         return self.logits.clone()
 
@@ -73,10 +84,20 @@ class StepPlan:
 
     def close(self) -> None:
         if self.handle is not None:
-            self.engine.lib.plan_free(self.handle)
+            try:
+                self.engine.lib.plan_free(self.handle)
+            except ReferenceError:            # the engine is gone already; the library outlives it
+                from ..csrc.lib import kernels
+                kernels().plan_free(self.handle)
             self.handle = None
         self.logits = None
         self.pool = None
+
+    def __del__(self) -> None:
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class StepPlans:
@@ -84,7 +105,7 @@ class StepPlans:
     of a varied load never come back, and a recording holds its buffers), and at most MAX_PLANS are kept."""
 
     def __init__(self, engine):
-        self.engine = engine
+        self.engine = weakref.proxy(engine)
         self.plans: "OrderedDict[Tuple, StepPlan]" = OrderedDict()
         self.seen: "OrderedDict[Tuple, int]" = OrderedDict()
         self.stats: Dict[str, int] = {"recorded": 0, "replayed": 0}
