@@ -43,8 +43,11 @@ int rb_rope_kv_write(const float* qkv, int qkv_terms, long long qkv_term_stride,
 int rb_swiglu(const float* gu, void* out, int out_dtype, int n_rows, int ff, void* stream);
 
 // C[M, N] = A[M, K] * W[N, K]^T with float32 accumulation; any sizes.
-int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dtype_out, int m, int n, int k,
-                    void* stream);
+// w_layout 0: W is N rows of K values.  1 (float32 with N % 16 == 0 and K % 128 == 0 only): fragment-major, blocks
+// of 16 rows x 16 depth values, 1 KB each, in the order [N / 16][K / 16]; inside a block the value of row r and
+// depth d lies at 4 * (16 * (d / 4) + r) + d % 4.  rb_place_rows writes either layout.
+int rb_gemm_generic(const void* a, const void* w, int w_layout, void* c, int dtype_in, int dtype_out, int m, int n,
+                    int k, void* stream);
 
 // C[M, N] = A[M, K] * W[N, K]^T, bfloat16 inputs on the matrix cores.
 //   epilogue 0: store C (float32 or bfloat16)
@@ -145,7 +148,8 @@ int rb_fill_normal(void* out, int dtype, long long n, unsigned long long key, do
 // row0 + (r / block) * period + r % block of dst [dst_rows, width].  block = n_rows places the rows
 // one after another from row0 (q, k, v in one matrix); block 16, period 32, row0 0 and 16 interleave
 // gate and up rows in blocks of 16.
-// dst_layout 1: dst is fragment-major (see rb_gemm_bf16; dst_rows % 16 == 0, width % 32 == 0).
+// dst_layout 1: dst is fragment-major for its type (bfloat16: see rb_gemm_bf16, dst_rows % 16 == 0, width % 32 == 0;
+// float32: see rb_gemm_generic, dst_rows % 16 == 0, width % 16 == 0).
 int rb_place_rows(const void* src, int src_dtype, void* dst, int dst_dtype, int dst_layout, long long n_rows,
                   long long width, long long dst_rows, long long row0, long long block, long long period, void* stream);
 

@@ -129,6 +129,138 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
     }
 }
 
+// Float32 operands, at most 64 tokens, K a multiple of 128 (the float32 path's decode step at the
+// widths of real models): bound by reading W once, and built like the bfloat16 product for few
+// tokens.  The float32 MFMA 16x16x4 (float32 inputs, products and sums): rows of W are the
+// matrix cores' row operand, the tokens their columns.  Lane l (row r = l % 16, group kq = l / 16)
+// loads 16 bytes of row r at depth 16 j + 4 kq and feeds its four values to four MFMAs; the tokens
+// are loaded the same way, so that an MFMA sums over the depths 16 j + 4 kq + i of its four groups
+// (which depth a group holds is free as long as both operands agree).  A stage is 128 depth values:
+// 8 loads of W per row tile, non-temporal (W is read once per step), all in flight while the stage
+// before is multiplied.  K is dealt to the waves of a workgroup in stages and their partial sums
+// meet in LDS in a fixed order.
+typedef __attribute__((ext_vector_type(4))) float gf_f32x4_t;
+
+template <int MB, int R, bool WF>
+__global__ __launch_bounds__(512) void gemm_f32_few_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                          float* __restrict__ c, int m, int n, int k) {
+  extern __shared__ float red[];      // [waves - 1][R * MB * 4][64]
+  constexpr int ACC = R * MB * 4;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+  const int r = lane & 15, kq = lane >> 4;
+  const int n0 = blockIdx.x * (16 * R);
+  gf_f32x4_t acc[R][MB];
+#pragma unroll
+  for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+    for (int cb = 0; cb < MB; ++cb) acc[rt][cb] = (gf_f32x4_t){0.f, 0.f, 0.f, 0.f};
+  // Where a lane finds its 4 values at depth ks + 16 j + 4 kq of row tile rt: wrow[rt] + (ks + 16 j) * WK.
+  // Rows [N, K]: the row's start + 4 kq, WK = 1.  Fragment-major (blocks of 16 rows x 16 depth values, 1 KB,
+  // the 16 bytes of lane l at 16 l): the tile's start + 4 lane, WK = 16; a wave's load is then 1 KB in a
+  // row, and W, read once per step, goes past the caches.
+  constexpr int WK = WF ? 16 : 1;
+  const float* wrow[R];
+#pragma unroll
+  for (int rt = 0; rt < R; ++rt) {
+    const int row = n0 + 16 * rt + r;
+    if (WF) wrow[rt] = w + (size_t)(n0 + 16 * rt < n ? n0 + 16 * rt : 0) * k + 4 * lane;
+    else wrow[rt] = w + (size_t)(row < n ? row : 0) * k + 4 * kq;        // rows beyond N: row 0, never stored
+  }
+  const float* xrow[MB];
+#pragma unroll
+  for (int cb = 0; cb < MB; ++cb) {
+    const int row = 16 * cb + r;
+    xrow[cb] = x + (size_t)(row < m ? row : 0) * k + 4 * kq;
+  }
+  // the K / 128 stages dealt to the waves as evenly as they go (the host launches no more waves than stages)
+  const int total = k / 128, base = total / n_waves, extra = total % n_waves;
+  const int stages = base + (wave < extra ? 1 : 0);
+  const int k_begin = 128 * (wave * base + (wave < extra ? wave : extra));
+  gf_f32x4_t a[R][8], b[MB][8];
+  auto load_stage = [&](int st) {
+    const int ks = k_begin + 128 * st;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int rt = 0; rt < R; ++rt)
+        a[rt][j] = WF ? __builtin_nontemporal_load(reinterpret_cast<const gf_f32x4_t*>(wrow[rt] + (size_t)(ks + 16 * j) * WK))
+                      : *reinterpret_cast<const gf_f32x4_t*>(wrow[rt] + ks + 16 * j);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int cb = 0; cb < MB; ++cb) b[cb][j] = *reinterpret_cast<const gf_f32x4_t*>(xrow[cb] + ks + 16 * j);
+  };
+  auto multiply_stage = [&]() {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+          for (int cb = 0; cb < MB; ++cb)
+            acc[rt][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[rt][j][i], b[cb][j][i], acc[rt][cb], 0, 0, 0);
+  };
+  load_stage(0);
+  for (int st = 1; st < stages; ++st) {
+    multiply_stage();
+    load_stage(st);
+  }
+  multiply_stage();
+
+  if (n_waves > 1) {
+    if (wave > 0) {
+      float* dst = red + (size_t)(wave - 1) * ACC * 64 + lane;
+#pragma unroll
+      for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+        for (int cb = 0; cb < MB; ++cb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dst[((rt * MB + cb) * 4 + i) * 64] = acc[rt][cb][i];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    for (int ww = 0; ww < n_waves - 1; ++ww) {
+      const float* src = red + (size_t)ww * ACC * 64 + lane;
+#pragma unroll
+      for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+        for (int cb = 0; cb < MB; ++cb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[rt][cb][i] += src[((rt * MB + cb) * 4 + i) * 64];
+    }
+  }
+  // lane l holds, for token 16 cb + l % 16, the rows n0 + 16 rt + 4 (l / 16) + i
+#pragma unroll
+  for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+    for (int cb = 0; cb < MB; ++cb) {
+      const int mm = 16 * cb + r, nn = n0 + 16 * rt + 4 * kq;
+      if (mm >= m) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (nn + i < n) c[(size_t)mm * n + nn + i] = acc[rt][cb][i];
+    }
+}
+
+static int g_f32_few = 1;
+extern "C" void rb_tune_f32_few(int on) { g_f32_few = on; }      // experiments only: 0 = the float32 product of few tokens (W as rows) on the vector units
+
+// One row tile per wave and at most 4 waves: measured at 1 to 16 tokens on the products of the 8B shape with W
+// fragment-major, two row tiles a wave lose everywhere but in the output matrix at 16 tokens (28,672 rows at
+// K = 4096, 8 tokens: 78 us against 93; 4,096 rows at K = 14336: 38 against 54), and 4 waves are as fast as 8
+// or faster (4,096 rows at K = 4096: 13.2 us against 14.4).
+template <int MB>
+static void launch_f32_few(const float* x, const float* w, bool w_frag, float* c, int m, int n, int k, hipStream_t s) {
+  int n_waves = k / 256;
+  if (n_waves < 1) n_waves = 1;
+  if (n_waves > 4) n_waves = 4;
+  const size_t lds = (size_t)(n_waves - 1) * MB * 4 * 64 * sizeof(float);
+  const int grid = (n + 15) / 16;
+  if (w_frag) gemm_f32_few_kernel<MB, 1, true><<<grid, 64 * n_waves, lds, s>>>(x, w, c, m, n, k);
+  else gemm_f32_few_kernel<MB, 1, false><<<grid, 64 * n_waves, lds, s>>>(x, w, c, m, n, k);
+}
+
 // Float32 operands and more than 16 tokens with K a multiple of 16 (the float32 path's
 // prefill): the float32 MFMA (v_mfma_f32_32x32x2_f32: float32 inputs, float32 products and
 // sums; no reduced-precision mode).  128 x 128 tiles, 16 deep, one wave per 64 x 64 piece.  W
@@ -142,6 +274,7 @@ typedef __attribute__((ext_vector_type(16))) float gf32x16_t;
 #define GM_K 16
 #define GM_LD (GM_T + 4)
 
+template <bool WF>
 __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                             float* __restrict__ c, int m, int n, int k) {
   __shared__ float ws[2][GM_K][GM_LD];
@@ -159,23 +292,37 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // staging: thread t loads, for q = t and t + 256, row q / 4 of the tile, depth values 4 (q % 4) .. + 3
+  // staging: thread t loads, for q = t and t + 256, row q / 4 of the tile, depth values 4 (q % 4) .. + 3;
+  // of a fragment-major W (blocks of 16 rows x 16 depth values, the 16 bytes of lane l at 16 l) the 16 bytes
+  // q % 64 of the tile's block q / 64: row 16 (q / 64) + q % 16, depth values 4 ((q % 64) / 16) .. + 3
   const float* wp[2];
   const float* xp[2];
+  int w_row[2], w_kk[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int q = tid + 256 * i;
-    int wr = n0 + q / 4, xr = m0 + q / 4;
-    if (wr > n - 1) wr = n - 1;            // rows beyond the matrix: a valid row, never stored
-    if (xr > m - 1) xr = m - 1;
-    wp[i] = w + (size_t)wr * k + 4 * (q % 4);
+    int xr = m0 + q / 4;
+    if (xr > m - 1) xr = m - 1;            // rows beyond the matrix: a valid row, never stored
     xp[i] = x + (size_t)xr * k + 4 * (q % 4);
+    if (WF) {
+      int tile = n0 / 16 + q / 64;
+      if (tile > n / 16 - 1) tile = n / 16 - 1;
+      w_row[i] = 16 * (q / 64) + q % 16;
+      w_kk[i] = 4 * ((q % 64) / 16);
+      wp[i] = w + (size_t)tile * 16 * k + 4 * (q % 64);
+    } else {
+      int wr = n0 + q / 4;
+      if (wr > n - 1) wr = n - 1;
+      w_row[i] = q / 4;
+      w_kk[i] = 4 * (q % 4);
+      wp[i] = w + (size_t)wr * k + 4 * (q % 4);
+    }
   }
   float4 wreg[2], xreg[2];
   auto load_tile = [&](int kt) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      wreg[i] = *reinterpret_cast<const float4*>(wp[i] + (size_t)kt * GM_K);
+      wreg[i] = *reinterpret_cast<const float4*>(wp[i] + (size_t)kt * (WF ? 256 : GM_K));
       xreg[i] = *reinterpret_cast<const float4*>(xp[i] + (size_t)kt * GM_K);
     }
   };
@@ -184,10 +331,10 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
     for (int i = 0; i < 2; ++i) {
       const int q = tid + 256 * i;
       const int row = q / 4, kk = 4 * (q % 4);
-      ws[buf][kk + 0][row] = wreg[i].x;
-      ws[buf][kk + 1][row] = wreg[i].y;
-      ws[buf][kk + 2][row] = wreg[i].z;
-      ws[buf][kk + 3][row] = wreg[i].w;
+      ws[buf][w_kk[i] + 0][w_row[i]] = wreg[i].x;
+      ws[buf][w_kk[i] + 1][w_row[i]] = wreg[i].y;
+      ws[buf][w_kk[i] + 2][w_row[i]] = wreg[i].z;
+      ws[buf][w_kk[i] + 3][w_row[i]] = wreg[i].w;
       xs[buf][kk + 0][row] = xreg[i].x;
       xs[buf][kk + 1][row] = xreg[i].y;
       xs[buf][kk + 2][row] = xreg[i].z;
@@ -231,12 +378,27 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
     }
 }
 
-extern "C" int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dtype_out, int m, int n,
-                               int k, void* stream) {
-  RB_RECORDED(rb_gemm_generic(a, w, c, dtype_in, dtype_out, m, n, k, stream));
+extern "C" int rb_gemm_generic(const void* a, const void* w, int w_layout, void* c, int dtype_in, int dtype_out, int m,
+                               int n, int k, void* stream) {
+  RB_RECORDED(rb_gemm_generic(a, w, w_layout, c, dtype_in, dtype_out, m, n, k, stream));
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_generic: bad sizes M=%d N=%d K=%d", m, n, k);
+  // a fragment-major W is float32 with N % 16 == 0 and K % 128 == 0: sizes that the two matrix-core kernels take
+  RB_REQUIRE(w_layout == 0 || (w_layout == 1 && dtype_in == RB_F32 && dtype_out == RB_F32 && n % 16 == 0 && k % 128 == 0),
+             "rb_gemm_generic: W layout %d with dtype %d, N=%d K=%d (fragment-major: float32, N %% 16 == 0, K %% 128 == 0)",
+             w_layout, dtype_in, n, k);
+  const bool w_frag = w_layout == 1;
   if (m == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  if (dtype_in == RB_F32 && dtype_out == RB_F32 && m <= 64 && k % 128 == 0 && (g_f32_few || w_frag)) {
+    const float* af = (const float*)a;
+    const float* wf = (const float*)w;
+    const int mb = (m + 15) / 16;
+    if (mb == 1) launch_f32_few<1>(af, wf, w_frag, (float*)c, m, n, k, s);
+    else if (mb == 2) launch_f32_few<2>(af, wf, w_frag, (float*)c, m, n, k, s);
+    else launch_f32_few<4>(af, wf, w_frag, (float*)c, m, n, k, s);
+    RB_LAUNCH_CHECK();
+    return 0;
+  }
   if (dtype_in == RB_F32 && dtype_out == RB_F32 && m <= 16 && k % 4 == 0) {
     const unsigned blocks = (unsigned)((n + 4 * GS_ROWS - 1) / (4 * GS_ROWS));
     const float* af = (const float*)a;
@@ -250,10 +412,12 @@ extern "C" int rb_gemm_generic(const void* a, const void* w, void* c, int dtype_
   if (dtype_in == RB_F32 && dtype_out == RB_F32 && m > 16 && k % GM_K == 0) {
     dim3 tiles((n + GM_T - 1) / GM_T, (m + GM_T - 1) / GM_T);
     RB_REQUIRE(tiles.y <= 65535, "rb_gemm_generic: M=%d too large for one launch", m);
-    gemm_f32_mfma_kernel<<<tiles, 256, 0, s>>>((const float*)a, (const float*)w, (float*)c, m, n, k);
+    if (w_frag) gemm_f32_mfma_kernel<true><<<tiles, 256, 0, s>>>((const float*)a, (const float*)w, (float*)c, m, n, k);
+    else gemm_f32_mfma_kernel<false><<<tiles, 256, 0, s>>>((const float*)a, (const float*)w, (float*)c, m, n, k);
     RB_LAUNCH_CHECK();
     return 0;
   }
+  RB_REQUIRE(!w_frag, "rb_gemm_generic: internal: a fragment-major W reached the kernels for rows");
   dim3 grid((n + GT - 1) / GT, (m + GT - 1) / GT);
   RB_REQUIRE(grid.y <= 65535, "rb_gemm_generic: M=%d too large for one launch", m);
   if (dtype_in == RB_F32 && dtype_out == RB_F32)

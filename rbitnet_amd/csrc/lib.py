@@ -129,7 +129,7 @@ class Kernels:
             "rb_add_rmsnorm": [_P, _P, _I, ctypes.c_longlong, _P, _F, _P, _I, _I, _P, _I, _P],
             "rb_rope_kv_write": [_P, _I, ctypes.c_longlong, _P, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
             "rb_swiglu": [_P, _P, _I, _I, _I, _P],
-            "rb_gemm_generic": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "rb_gemm_generic": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
             "rb_gemm_bf16": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _P, _P],
             "rb_gemm_bf16_few": [_P, _P, _F, _P, _P, _I, _P, _I, _I, _P, _P, _P, _I, _I, _I, _P],
             "rb_gemm_bf16_few_ok": [_I, _I, _I],
@@ -247,14 +247,15 @@ class Kernels:
         _check(out, "out")
         self._ok(self._lib.rb_swiglu(_ptr(gu), _ptr(out), dtype_code(out.dtype), n, ff, self._stream()))
 
-    def gemm_generic(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor) -> None:
+    def gemm_generic(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, w_frag: bool = False) -> None:
+        """w_frag: w [N, K] (float32) is stored fragment-major (`place_rows(..., frag=True)` writes that)."""
         m, k = a.shape
         n = w.shape[0]
         _check(a, "a")
         _check(w, "w", a.dtype, (n, k))
         _check(c, "c", None, (m, n))
-        self._ok(self._lib.rb_gemm_generic(_ptr(a), _ptr(w), _ptr(c), dtype_code(a.dtype), dtype_code(c.dtype),
-                                           m, n, k, self._stream()))
+        self._ok(self._lib.rb_gemm_generic(_ptr(a), _ptr(w), int(bool(w_frag)), _ptr(c), dtype_code(a.dtype),
+                                           dtype_code(c.dtype), m, n, k, self._stream()))
 
     def gemm_bf16(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = 0,
                   w_frag: bool = False) -> None:

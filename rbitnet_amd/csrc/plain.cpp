@@ -69,13 +69,14 @@ float sum_terms(const float* p, int n_terms, size_t stride) {
 }
 
 // Where element (row, col) of W [N, K] lies.  layout 0: rows.  layout 1: fragment-major, blocks of
-// 16 rows x 32 columns in the order [N / 16][K / 32]; inside a block the value of row r, column q
-// at 8 * (16 * (q / 8) + r) + q % 8.
-size_t w_at(int layout, long long n_cols, long long row, long long col) {
+// 16 rows x 4 E columns (E = values of the type in 16 bytes: 8 bfloat16, 4 float32) in the order
+// [N / 16][K / (4 E)]; inside a block the value of row r, column q at E * (16 * (q / E) + r) + q % E.
+size_t w_at(int layout, int dtype, long long n_cols, long long row, long long col) {
   if (layout == 0) return (size_t)(row * n_cols + col);
-  const long long block = (row / 16) * (n_cols / 32) + col / 32;
-  const long long r = row % 16, q = col % 32;
-  return (size_t)(block * 512 + 8 * (16 * (q / 8) + r) + q % 8);
+  const long long e = dtype == F32 ? 4 : 8;
+  const long long block = (row / 16) * (n_cols / (4 * e)) + col / (4 * e);
+  const long long r = row % 16, q = col % (4 * e);
+  return (size_t)(block * 64 * e + e * (16 * (q / e) + r) + q % e);
 }
 
 double silu(double v) { return v / (1.0 + exp(-v)); }      // model.rs:116-120
@@ -144,7 +145,7 @@ void product(const void* a, int a_dtype, const int32_t* rows, const void* w, int
     for (int kk = 0; kk < k; ++kk) ar[kk] = load(a, a_dtype, src * k + kk);
     for (int j = 0; j < n; ++j) {
       double acc = 0.0;
-      for (int kk = 0; kk < k; ++kk) acc += ar[kk] * load(w, w_dtype, w_at(w_layout, k, j, kk));
+      for (int kk = 0; kk < k; ++kk) acc += ar[kk] * load(w, w_dtype, w_at(w_layout, w_dtype, k, j, kk));
       c[(size_t)i * n + j] = acc;
     }
   }
@@ -263,11 +264,14 @@ int rbp_swiglu(const float* gu, void* out, int out_dtype, int n_rows, int ff, vo
 }
 
 // C[M, N] = A[M, K] W[N, K]^T  (model.rs:67-91)
-int rbp_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dtype_out, int m, int n, int k, void*) {
+int rbp_gemm_generic(const void* a, const void* w, int w_layout, void* c, int dtype_in, int dtype_out, int m, int n,
+                     int k, void*) {
   REQUIRE(dtype_ok(dtype_in) && dtype_ok(dtype_out), "rbp_gemm_generic: unknown dtype %d / %d", dtype_in, dtype_out);
   REQUIRE(m >= 0 && n > 0 && k > 0, "rbp_gemm_generic: bad sizes M=%d N=%d K=%d", m, n, k);
+  REQUIRE(w_layout == 0 || (w_layout == 1 && dtype_in == F32 && n % 16 == 0 && k % 128 == 0),
+          "rbp_gemm_generic: W layout %d with dtype %d, N=%d K=%d", w_layout, dtype_in, n, k);
   std::vector<double> acc;
-  product(a, dtype_in, nullptr, w, dtype_in, 0, m, n, k, acc);
+  product(a, dtype_in, nullptr, w, dtype_in, w_layout, m, n, k, acc);
   for (size_t i = 0; i < acc.size(); ++i) store(c, dtype_out, i, acc[i]);
   return 0;
 }
@@ -442,13 +446,13 @@ int rbp_place_rows(const void* src, int src_dtype, void* dst, int dst_dtype, int
                    long long width, long long dst_rows, long long row0, long long block, long long period, void*) {
   REQUIRE(dtype_ok(src_dtype) && dtype_ok(dst_dtype), "rbp_place_rows: unknown dtype %d / %d", src_dtype, dst_dtype);
   REQUIRE(block > 0 && period >= block, "rbp_place_rows: block %lld, period %lld", block, period);
-  REQUIRE(dst_layout == 0 || (dst_layout == 1 && dst_rows % 16 == 0 && width % 32 == 0),
+  REQUIRE(dst_layout == 0 || (dst_layout == 1 && dst_rows % 16 == 0 && width % (dst_dtype == F32 ? 16 : 32) == 0),
           "rbp_place_rows: layout %d for %lld rows of %lld", dst_layout, dst_rows, width);
   for (long long r = 0; r < n_rows; ++r) {
     const long long to = row0 + (r / block) * period + r % block;
     REQUIRE(to >= 0 && to < dst_rows, "rbp_place_rows: row %lld goes to %lld of %lld", r, to, dst_rows);
     for (long long j = 0; j < width; ++j)
-      store(dst, dst_dtype, w_at(dst_layout, width, to, j), load(src, src_dtype, (size_t)(r * width + j)));
+      store(dst, dst_dtype, w_at(dst_layout, dst_dtype, width, to, j), load(src, src_dtype, (size_t)(r * width + j)));
   }
   return 0;
 }

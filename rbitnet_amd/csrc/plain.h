@@ -31,8 +31,8 @@ int rbp_rope_kv_write(const float* qkv, int qkv_terms, long long qkv_term_stride
                       const int32_t* tok_seq, const int32_t* block_table, int bt_stride, int n_tokens, int n_heads,
                       int n_kv_heads, int head_dim, void* stream);
 int rbp_swiglu(const float* gu, void* out, int out_dtype, int n_rows, int ff, void* stream);
-int rbp_gemm_generic(const void* a, const void* w, void* c, int dtype_in, int dtype_out, int m, int n, int k,
-                     void* stream);
+int rbp_gemm_generic(const void* a, const void* w, int w_layout, void* c, int dtype_in, int dtype_out, int m, int n,
+                     int k, void* stream);
 int rbp_gemm_bf16(const void* a, const void* w, int w_layout, void* c, int dtype_out, int epilogue, int m, int n, int k,
                   float* workspace, void* stream);
 int rbp_gemm_bf16_few(const void* a, const float* squares_in, float eps, const int32_t* rows, const void* w,

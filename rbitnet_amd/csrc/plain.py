@@ -48,7 +48,7 @@ class PlainKernels:
             "rbp_add_rmsnorm": [_P, _P, _I, _LL, _P, _F, _P, _I, _I, _P, _I, _P],
             "rbp_rope_kv_write": [_P, _I, _LL, _P, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
             "rbp_swiglu": [_P, _P, _I, _I, _I, _P],
-            "rbp_gemm_generic": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "rbp_gemm_generic": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
             "rbp_gemm_bf16": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _P, _P],
             "rbp_gemm_bf16_few": [_P, _P, _F, _P, _P, _I, _P, _I, _I, _P, _P, _P, _I, _I, _I, _P],
             "rbp_attention_generic": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
@@ -90,10 +90,10 @@ class PlainKernels:
         n, ff = out.shape
         self._ok(self._lib.rbp_swiglu(_ptr(gu), _ptr(out), _code(out.dtype), n, ff, None))
 
-    def gemm_generic(self, a, w, c) -> None:
+    def gemm_generic(self, a, w, c, w_frag: bool = False) -> None:
         m, k = a.shape
-        self._ok(self._lib.rbp_gemm_generic(_ptr(a), _ptr(w), _ptr(c), _code(a.dtype), _code(c.dtype), m, w.shape[0], k,
-                                            None))
+        self._ok(self._lib.rbp_gemm_generic(_ptr(a), _ptr(w), int(bool(w_frag)), _ptr(c), _code(a.dtype), _code(c.dtype),
+                                            m, w.shape[0], k, None))
 
     def gemm_bf16(self, a, w, c, epilogue: int = 0, w_frag: bool = False) -> None:
         m, k = a.shape

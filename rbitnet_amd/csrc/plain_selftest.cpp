@@ -88,7 +88,7 @@ int main() {
     OK(rbp_gemm_bf16(a.data(), wf.data(), 1, c1.data(), 0, 0, m, n, k, nullptr, nullptr));
     CHECK(memcmp(c0.data(), c1.data(), c0.size() * 4) == 0, "rows and fragment-major W give the same product");
     std::vector<float> cg(m * n);
-    OK(rbp_gemm_generic(a.data(), w.data(), cg.data(), 1, 0, m, n, k, nullptr));
+    OK(rbp_gemm_generic(a.data(), w.data(), 0, cg.data(), 1, 0, m, n, k, nullptr));
     CHECK(memcmp(c0.data(), cg.data(), c0.size() * 4) == 0, "the generic product is the same product");
     std::vector<uint16_t> gated(m * n / 2);
     OK(rbp_gemm_bf16(a.data(), w.data(), 0, gated.data(), 1, 1, m, n, k, nullptr, nullptr));
@@ -118,8 +118,18 @@ int main() {
     std::vector<float> eye(e * e, 0.f), xin(2 * e), xout(2 * e);
     for (int i = 0; i < e; ++i) eye[i * e + i] = 1.f;
     for (auto& v : xin) v = noise(seed);
-    OK(rbp_gemm_generic(xin.data(), eye.data(), xout.data(), 0, 0, 2, e, e, nullptr));
+    OK(rbp_gemm_generic(xin.data(), eye.data(), 0, xout.data(), 0, 0, 2, e, e, nullptr));
     CHECK(memcmp(xin.data(), xout.data(), xin.size() * 4) == 0, "a product against the identity");
+    // float32 W fragment-major: the same product
+    const int fn = 32, fk = 128;
+    std::vector<float> fw(fn * fk), fwf(fn * fk), fx(3 * fk), f0(3 * fn), f1(3 * fn);
+    for (auto& v : fw) v = noise(seed);
+    for (auto& v : fx) v = noise(seed);
+    OK(rbp_place_rows(fw.data(), 0, fwf.data(), 0, 1, fn, fk, fn, 0, fn, fn, nullptr));
+    OK(rbp_gemm_generic(fx.data(), fw.data(), 0, f0.data(), 0, 0, 3, fn, fk, nullptr));
+    OK(rbp_gemm_generic(fx.data(), fwf.data(), 1, f1.data(), 0, 0, 3, fn, fk, nullptr));
+    CHECK(memcmp(f0.data(), f1.data(), f0.size() * 4) == 0, "float32 rows and fragment-major W give the same product");
+    CHECK(rbp_gemm_generic(fx.data(), fwf.data(), 1, f1.data(), 0, 0, 3, fn, 64, nullptr) != 0, "fragment-major float32 needs K % 128 == 0");
   }
   // ---- rotation and cache write, attention over pages, every form of it
   {

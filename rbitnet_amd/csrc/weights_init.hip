@@ -127,9 +127,12 @@ __global__ __launch_bounds__(256) void place_rows_kernel(const S* __restrict__ s
        i += (long long)gridDim.x * blockDim.x) {
     const long long r = i / width, c = i - r * width;
     const long long d = row0 + (r / block) * period + r % block;
-    // fragment-major: blocks of 16 rows x 32 columns in the order [rows / 16][width / 32]; inside a
-    // block the value of row r, column q lies at 8 * (16 * (q / 8) + r) + q % 8
-    const long long at = frag ? ((d / 16) * (width / 32) + c / 32) * 512 + (16 * ((c % 32) / 8) + d % 16) * 8 + c % 8
+    // fragment-major: blocks of 16 rows x 4 E columns (1 KB; E = the values of the destination's type
+    // in 16 bytes: 8 bfloat16, 4 float32) in the order [rows / 16][width / (4 E)]; inside a block the
+    // value of row r, column q lies at E * (16 * (q / E) + r) + q % E
+    constexpr long long E = 16 / sizeof(T);
+    const long long at = frag ? ((d / 16) * (width / (4 * E)) + c / (4 * E)) * (64 * E) +
+                                    (16 * ((c % (4 * E)) / E) + d % 16) * E + c % E
                               : d * width + c;
     Num<T>::store(dst + at, Num<S>::load(src + i));
   }
@@ -161,7 +164,7 @@ extern "C" int rb_fill_normal(void* out, int dtype, long long n, unsigned long l
 extern "C" int rb_place_rows(const void* src, int src_dtype, void* dst, int dst_dtype, int dst_layout,
                              long long n_rows, long long width, long long dst_rows, long long row0, long long block,
                              long long period, void* stream) {
-  RB_REQUIRE(dst_layout == 0 || (dst_layout == 1 && dst_rows % 16 == 0 && width % 32 == 0),
+  RB_REQUIRE(dst_layout == 0 || (dst_layout == 1 && dst_rows % 16 == 0 && width % (dst_dtype == RB_F32 ? 16 : 32) == 0),
              "rb_place_rows: layout %d of a destination of %lld rows of %lld", dst_layout, dst_rows, width);
   RB_REQUIRE(n_rows >= 0 && width > 0 && block > 0 && period >= block && row0 >= 0,
              "rb_place_rows: bad sizes (rows %lld, width %lld, block %lld, period %lld, first row %lld)", n_rows, width,

@@ -24,10 +24,11 @@ GATE_BLOCK = 16     # rows per block when gate and up rows are interleaved for t
 
 class Matrix:
     """A weight matrix [N, K] as the product kernels read it.  `data` holds its N x K values, as N
-    rows, or, `frag`, fragment-major: blocks of 16 rows x 32 columns of 1 KB in the order
-    [N / 16][K / 32], laid out as the matrix cores' row operand, so that a wave reads 1 KB in a row
-    per load and a decode step streams W past the caches (6.0-6.8 TB/s against 5.3-5.8 for rows).
-    Only bfloat16 matrices with N % 16 == 0 and K % 64 == 0 are stored so; `pack_rows` decides."""
+    rows, or, `frag`, fragment-major: blocks of 1 KB (16 rows x 32 bfloat16 or 16 float32 columns) in
+    the order [N / 16][K / columns], laid out as the matrix cores' row operand, so that a wave reads
+    1 KB in a row per load and a decode step streams W past the caches (bfloat16: 6.0-6.8 TB/s against
+    5.3-5.8 for rows).  bfloat16 matrices with N % 16 == 0 and K % 64 == 0 and float32 ones with
+    N % 16 == 0 and K % 128 == 0 are stored so; `pack_rows` decides."""
 
     def __init__(self, data: torch.Tensor, frag: bool = False):
         self.data, self.frag = data, bool(frag)
@@ -39,6 +40,10 @@ def _data(w):
 
 
 def fragment_major_ok(dtype: torch.dtype, n: int, k: int) -> bool:
+    """bfloat16: the matrix-core products read either layout when N % 16 == 0 and K % 64 == 0.  float32:
+    with N % 16 == 0 and K % 128 == 0 every step's product runs on a kernel that reads it."""
+    if dtype == torch.float32:
+        return n % 16 == 0 and k % 128 == 0
     return dtype == torch.bfloat16 and n % 16 == 0 and k % 64 == 0
 
 
@@ -87,11 +92,11 @@ def linear(lib, x, w, out_dtype: torch.dtype) -> torch.Tensor:
     if uses_matrix_cores(x.dtype, k):
         lib.gemm_bf16(x, wd, out, 0, w_frag=frag)
     else:
-        if frag:
-            raise KernelError("a fragment-major matrix is for the matrix-core products only")
+        if frag and x.dtype != torch.float32:
+            raise KernelError("a fragment-major bfloat16 matrix is for the matrix-core products only")
         if x.dtype == torch.float32 and out_dtype != torch.float32:
             raise KernelError("a float32 product has a float32 result")
-        lib.gemm_generic(x, wd, out)
+        lib.gemm_generic(x, wd, out, w_frag=frag)
     return out
 
 

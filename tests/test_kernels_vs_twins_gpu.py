@@ -129,6 +129,45 @@ def test_gemm_generic(lib, twin, m, n, k):
         _close(*res[2], what=f"generic product {dtype}")
 
 
+@pytest.mark.parametrize("m", [1, 7, 16, 17, 33, 64])
+@pytest.mark.parametrize("n,k", [(1000, 128), (4096, 512), (8208, 256), (160, 4096 + 128), (28672, 384)])
+def test_gemm_float32_of_few_tokens(lib, twin, m, n, k):
+    """The float32 product for up to 64 tokens on the float32 MFMA (K a multiple of 128): row counts
+    that fill no tile of 16, every number of token blocks, one and two row tiles a workgroup, K in 1 to
+    8 waves with uneven shares, and the same product on the vector units."""
+    g = _gen(m * 13 + n + k)
+    a, w = torch.randn(m, k, generator=g), torch.randn(n, k, generator=g)
+    res = _both(lib, twin, "gemm_generic", [a, w, torch.full((m, n), float("nan"))], [2])
+    _close(*res[2], what="float32 product of few tokens")
+    lib._lib.rb_tune_f32_few(0)
+    try:
+        other = torch.full((m, n), float("nan"), device=DEV)
+        lib.gemm_generic(a.to(DEV), w.to(DEV), other)
+    finally:
+        lib._lib.rb_tune_f32_few(1)
+    _close(other, res[2][1], what="float32 product of few tokens on the vector units")
+    if n % 16 == 0:
+        wf = torch.empty_like(w)
+        twin.place_rows(w, wf, frag=True)
+        frag = _both(lib, twin, "gemm_generic", [a, wf, torch.full((m, n), float("nan"))], [2], w_frag=True)
+        _close(*frag[2], what="float32 product of few tokens, W fragment-major")
+        assert torch.equal(frag[2][0], res[2][0])          # the same sums in the same order
+
+
+@pytest.mark.parametrize("m,n,k", [(65, 992, 256), (200, 4096, 128), (300, 160, 1024)])
+def test_gemm_float32_of_many_tokens_with_fragment_major_weights(lib, twin, m, n, k):
+    """The float32 MFMA tiles reading W as rows and fragment-major: the same bits, and the twin's product."""
+    g = _gen(m + n + k)
+    a, w = torch.randn(m, k, generator=g), torch.randn(n, k, generator=g)
+    wf = torch.empty_like(w)
+    twin.place_rows(w, wf, frag=True)
+    rows = _both(lib, twin, "gemm_generic", [a, w, torch.full((m, n), float("nan"))], [2])
+    frag = _both(lib, twin, "gemm_generic", [a, wf, torch.full((m, n), float("nan"))], [2], w_frag=True)
+    _close(*rows[2], what="float32 tiles, W as rows")
+    _close(*frag[2], what="float32 tiles, W fragment-major")
+    assert torch.equal(frag[2][0], rows[2][0]) and torch.equal(frag[2][1], rows[2][1])
+
+
 @pytest.mark.parametrize("m", [1, 8, 16, 17, 64, 200, 600])
 @pytest.mark.parametrize("n,k", [(992, 1024), (4096, 512), (1376, 200), (160, 4096)])
 def test_gemm_bf16(lib, twin, m, n, k):
@@ -197,16 +236,30 @@ def _paged(g, past, q_lens, hk, d, dtype, n_pages=24):
 
 @pytest.mark.parametrize("dtype", [F32, BF])
 @pytest.mark.parametrize("window", [0, 50])
-def test_attention_generic(lib, twin, dtype, window):
-    g = _gen(20 + window)
-    hq, hk, d = 6, 2, 24
+@pytest.mark.parametrize("d", [24, 18, 128, 256])
+def test_attention_generic(lib, twin, dtype, window, d):
+    """Head sizes that are multiples of 4 (16-byte loads, the lanes in groups of 8, 32 and 64) and one that is
+    not (the scalar kernel), which is also run on a size the other kernel takes."""
+    g = _gen(20 + window + d)
+    hq, hk = 6, 2
     past, q_lens = [63, 0, 130, 0], [3, 1, 70, 64]
     kp, vp, bt, tok_pos, tok_seq = _paged(g, past, q_lens, hk, d, dtype)
     n = int(tok_pos.numel())
     q = torch.randn(n, hq, d, generator=g).to(dtype)
-    res = _both(lib, twin, "attention_generic", [q, kp, vp, torch.empty(n, hq * d, dtype=dtype), tok_pos, tok_seq, bt,
-                                                 hq, hk, d, d ** -0.5, window], [3])
+    args = [q, kp, vp, torch.empty(n, hq * d, dtype=dtype), tok_pos, tok_seq, bt, hq, hk, d, d ** -0.5, window]
+    res = _both(lib, twin, "attention_generic", args, [3])
     _close(*res[3], what="attention")
+    # few tokens: 8 waves to a (token, head), which merge their states
+    few = [a[-2:].contiguous() if isinstance(a, torch.Tensor) and a.shape[:1] == (n,) else a for a in args]
+    res = _both(lib, twin, "attention_generic", few, [3])
+    _close(*res[3], what="attention of two tokens")
+    if d == 24:
+        lib._lib.rb_tune_attention_vec(0)
+        try:
+            res = _both(lib, twin, "attention_generic", args, [3])
+        finally:
+            lib._lib.rb_tune_attention_vec(1)
+        _close(*res[3], what="attention, scalar kernel")
 
 
 @pytest.mark.parametrize("d", [64, 128])
@@ -276,8 +329,6 @@ def test_place_rows(lib, twin):
     src = torch.randn(48, 64, generator=g)
     for dtype in (F32, BF):
         for frag in (False, True):
-            if frag and dtype != BF:
-                continue
             args = lambda row0, block, period: [src.to(dtype), torch.zeros(128, 64, dtype=dtype), row0, block, period]
             for a in (args(0, None, None), args(32, None, None), args(16, 16, 32)):
                 res = _both(lib, twin, "place_rows", a, [1], frag=frag)
