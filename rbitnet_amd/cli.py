@@ -4,10 +4,12 @@ variables as its `#[arg(long, env = ...)]` do; failures print `error: ...` and e
 with 1, main.rs:300-303).
 
     rbitnet generate --model DIR --prompt-ids 1,2,3 [--prompt-ids 4,5 ...] [--max-tokens 256]
-                     [--temperature 0.7] [--seed 0] [--stop-token-ids 2,7] [--dtype bfloat16]
+                     [--temperature 0.7] [--seed 0] [--stop-token-ids 2,7] [--add-bos] [--dtype bfloat16]
     rbitnet random   --config config.json --out DIR [--seed 42] [--init-std 0.02] [--norm-std 0.02]
     rbitnet inspect  DIR_OR_FILE
-    rbitnet replay   --model DIR --dtype D --out DIR --max-tokens N   < trace.jsonl
+    rbitnet replay   --model DIR --dtype D --out DIR --max-tokens N   < trace.jsonl        (steps)
+    rbitnet replay   --model DIR --dtype D --out DIR --max-tokens N --requests FILE --mode whole|tail|batched
+                     [--batch-size B]                                                     (whole requests)
     rbitnet bench    [--steps K] [--warmup W] [--batch B] [--layers L] [--no-points]
 
 Environment, as the reference's engine reads it (crates/bitnet-core/src/inference.rs:16-41):
@@ -94,7 +96,12 @@ def cmd_generate(args) -> int:
                 prompts.append(json.loads(line) if line.startswith("[") else _ids(line))
     if not prompts:
         raise ConfigError("no prompt given (--prompt-ids or --prompt-file)")
-    engine = _engine(args, [max(1, len(p)) for p in prompts], args.max_tokens)
+    engine = _engine(args, [len(p) + 1 for p in prompts], args.max_tokens)
+    if args.add_bos:
+        bos = engine.spec.bos_token_id
+        if bos is None:
+            raise ConfigError("--add-bos: the model's configuration names no BOS token (bos_token_id)")
+        prompts = [[int(bos)] + p for p in prompts]
     stop = _ids(args.stop_token_ids) if args.stop_token_ids else None
     results = engine.generate(prompts, max_tokens=args.max_tokens, temperature=args.temperature, seed=args.seed,
                               stop_token_ids=stop)
@@ -156,6 +163,14 @@ def cmd_inspect(args) -> int:
 def cmd_replay(args) -> int:
     from .engine import Engine
     from .replay import replay
+    if args.requests:
+        from .replay import replay_requests
+        with open(args.requests) as f:
+            requests = [json.loads(line) for line in f if line.strip()]
+        engine = Engine.load_path(args.model, dtype=args.dtype, max_tokens=args.max_tokens,
+                                  max_batch=max(1, args.batch_size))
+        replay_requests(engine, requests, args.mode, args.out, batch_size=args.batch_size)
+        return 0
     engine = Engine.load_path(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
     replay(engine, sys.stdin, args.out)
     return 0
@@ -182,6 +197,7 @@ def build_parser() -> argparse.ArgumentParser:
     g.add_argument("--temperature", type=float, default=0.7)
     g.add_argument("--seed", type=int, default=0, help="seed of the sampler")
     g.add_argument("--stop-token-ids", help="comma-separated ids that end a sequence (besides the model's EOS)")
+    g.add_argument("--add-bos", action="store_true", help="put the model's BOS token before every prompt")
     g.add_argument("--max-batch", type=int, default=8, help="sequences that run together")
     g.add_argument("--max-seq-len", type=int, default=None, help="most tokens a sequence may hold")
     g.set_defaults(fn=cmd_generate)
@@ -204,6 +220,11 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     p.add_argument("--out", required=True)
     p.add_argument("--max-tokens", type=int, required=True)
+    p.add_argument("--requests", help="a file of whole requests, one JSON object a line: {\"id\": .., \"tokens\": [..]}; "
+                                      "without it, steps are read from standard input")
+    p.add_argument("--mode", default="whole", choices=["whole", "tail", "batched"],
+                   help="how --requests are cut into steps (the logits must not depend on it)")
+    p.add_argument("--batch-size", type=int, default=4, help="requests that run together in --mode batched")
     p.set_defaults(fn=cmd_replay)
 
     b = sub.add_parser("bench", help="decode and prefill throughput at the Llama-3-8B shape (one JSON line)",

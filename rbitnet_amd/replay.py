@@ -63,6 +63,67 @@ def replay(engine, lines: IO[str], out_dir: str, log: IO[str] = sys.stdout) -> i
     return n
 
 
+def replay_requests(engine, requests, mode: str, out_dir: str, batch_size: int = 1, tail: int = 32) -> Dict[str, str]:
+    """Whole requests instead of steps: `requests` is a list of {"id", "tokens"[, "prefill"]}; every
+    request's logits at all its positions go to `<out>/<id>.npy` (float32 [T, vocab]) and an
+    `index.json` names them.  The mode says how the tokens are cut into steps, which must not
+    change the logits beyond rounding:
+      whole    each request alone, all tokens in one step;
+      tail     each request alone, all but the last `tail` tokens in one step, the rest one by one;
+      batched  `batch_size` requests at a time in file order: their first tokens (all but the last
+               `tail`, or the request's own "prefill" count) in one step of unequal lengths, then one
+               token per request still running; a request that has run out leaves and frees its
+               slot, and the next group starts in the same slots."""
+    import numpy as np
+    import torch
+    if mode not in ("whole", "tail", "batched"):
+        raise RbitnetError(f"unknown replay mode {mode!r} (whole, tail, batched)")
+    os.makedirs(out_dir, exist_ok=True)
+    reqs = [(str(r["id"]), [int(t) for t in r["tokens"]], r.get("prefill")) for r in requests]
+    for rid, toks, _ in reqs:
+        if not toks:
+            raise RbitnetError(f"request {rid!r} has no tokens")
+    index: Dict[str, str] = {}
+    group = max(1, int(batch_size)) if mode == "batched" else 1
+    for g0 in range(0, len(reqs), group):
+        batch = reqs[g0:g0 + group]
+        slots = [engine.alloc_slot() for _ in batch]
+        heads = []
+        for _, toks, prefill in batch:
+            if mode == "whole":
+                heads.append(len(toks))
+            elif prefill is not None and mode == "batched":
+                heads.append(max(1, min(int(prefill), len(toks))))
+            else:
+                heads.append(max(1, len(toks) - tail) if len(toks) > tail else 1)
+        rows = [[] for _ in batch]
+        logits = engine.step([(s, toks[:h]) for s, (_, toks, _), h in zip(slots, batch, heads)], "all")
+        off = 0
+        for i, h in enumerate(heads):
+            rows[i].append(logits[off:off + h].to("cpu"))
+            off += h
+        done = list(heads)
+        live = [i for i in range(len(batch)) if done[i] < len(batch[i][1])]
+        for i in range(len(batch)):
+            if i not in live:
+                engine.free_slot(slots[i])
+        while live:
+            logits = engine.step([(slots[i], [batch[i][1][done[i]]]) for i in live], "last").to("cpu")
+            for row, i in enumerate(live):
+                rows[i].append(logits[row:row + 1])
+                done[i] += 1
+            for i in [i for i in live if done[i] >= len(batch[i][1])]:
+                engine.free_slot(slots[i])
+            live = [i for i in live if done[i] < len(batch[i][1])]
+        for i, (rid, toks, _) in enumerate(batch):
+            name = f"{rid}.npy"
+            np.save(os.path.join(out_dir, name), torch.cat(rows[i]).numpy().astype("<f4", copy=False))
+            index[rid] = name
+    with open(os.path.join(out_dir, "index.json"), "w") as f:
+        json.dump({"mode": mode, "requests": index}, f, indent=1)
+    return index
+
+
 def main(argv: Optional[list] = None) -> int:
     ap = argparse.ArgumentParser(prog="trace_run", description="Replay a trace of token ids and write logits.")
     ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")

@@ -146,6 +146,28 @@ def test_command_line_random_weights_and_toy_mode(tmp_path):
     assert "need --config" in r.stderr
 
 
+def test_command_line_add_bos(tmp_path):
+    """--add-bos puts the configuration's BOS id before every prompt: the same tokens as the prompt
+    given with that id in front; a configuration without one refuses the flag."""
+    cfg = dict(TINY_B, bos_token_id=11)
+    cfg_path = str(tmp_path / "config.json")
+    with open(cfg_path, "w") as f:
+        json.dump(cfg, f)
+    common = ["generate", "--random", "--config", cfg_path, "--max-tokens", "6", "--temperature", "0", "--dtype", "float32"]
+    with_flag = [json.loads(line) for line in
+                 _cli(common + ["--add-bos", "--prompt-ids", "5,6", "--prompt-ids", "9"]).stdout.strip().splitlines()]
+    by_hand = [json.loads(line) for line in
+               _cli(common + ["--prompt-ids", "11,5,6", "--prompt-ids", "11,9"]).stdout.strip().splitlines()]
+    assert with_flag == by_hand and [r["prompt_tokens"] for r in with_flag] == [3, 2]
+    without = [json.loads(line) for line in _cli(common + ["--prompt-ids", "5,6", "--prompt-ids", "9"]).stdout.strip().splitlines()]
+    assert [r["prompt_tokens"] for r in without] == [2, 1]
+    none = {k: v for k, v in TINY_B.items() if k != "bos_token_id"}
+    with open(cfg_path, "w") as f:
+        json.dump(none, f)
+    r = _cli(common + ["--add-bos", "--prompt-ids", "5"], expect=1)
+    assert "bos_token_id" in r.stderr
+
+
 def test_kernel_times_behind_an_environment_flag(tmp_path):
     """RBITNET_KERNEL_TIMES=1: a table of GPU time per kernel wrapper on standard error when the
     process ends; the tokens are the ones a run without it generates."""

@@ -93,6 +93,35 @@ def test_replay_whole_tail_and_batched(name, dtype, tmp_path):
     rp.close()
 
 
+@pytest.mark.parametrize("mode", ["whole", "tail", "batched"])
+def test_replay_of_whole_requests(mode, tmp_path):
+    """`rbitnet replay --requests`: a file of requests, every position's logits per request as .npy
+    and an index; the three ways of cutting give the plain implementation's logits.  Five requests in
+    groups of two: the last group is smaller, and every group takes the slots the one before freed."""
+    name, dtype = "B", "float32"
+    lengths = [3, 50, 33, 70, 34]
+    reqs = {f"q{i}": tokens_for(name, n, 40 + i) for i, n in enumerate(lengths)}
+    trace = tmp_path / "requests.jsonl"
+    with open(trace, "w") as f:
+        for i, (k, v) in enumerate(reqs.items()):
+            rec = {"id": k, "tokens": v}
+            if i == 3:
+                rec["prefill"] = 11                      # its own cut, used by the batched mode
+            f.write(json.dumps(rec) + "\n")
+    out = tmp_path / "out"
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "rbitnet"), "replay", "--model", model_folder(name),
+                        "--dtype", dtype, "--out", str(out), "--max-tokens", str(64 * 4), "--requests", str(trace),
+                        "--mode", mode, "--batch-size", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    with open(out / "index.json") as f:
+        index = json.load(f)
+    assert index["mode"] == mode and sorted(index["requests"]) == sorted(reqs)
+    for k, toks in reqs.items():
+        got = torch.from_numpy(np.load(out / index["requests"][k]))
+        assert got.dtype == torch.float32 and got.shape == (len(toks), CONFIGS[name][0]["vocab_size"])
+        assert max_err(got, plain_logits(name, tuple(toks))) < TOL[dtype], (mode, k)
+
+
 def test_replay_reports_errors(tmp_path):
     out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", str(tmp_path),
                           "--dtype", "float32", "--out", str(tmp_path / "o"), "--max-tokens", "64"],
