@@ -222,6 +222,34 @@ def probe(lib, device) -> dict:
     return out
 
 
+def load_probe(cfg, tokens: int, reps: int = 12) -> None:
+    """For a profiler that counts cycles (`rocprofv3 --pmc GRBM_GUI_ACTIVE SQ_VALU_MFMA_BUSY_CYCLES --kernel-trace`):
+    the MFMA probe, the gated product of the named shape with `tokens` tokens and the same product with 8 tokens,
+    `reps` launches of each in a row.  GRBM_GUI_ACTIVE of a launch over its duration is the clock the GPU ran
+    at, which under a product of many tokens is far below the one the nominal peak is quoted at."""
+    import torch
+    from .csrc.lib import kernels
+    lib = kernels()
+    dev, bf = "cuda:0", torch.bfloat16
+    sink = torch.zeros(1 << 20, device=dev)
+    for _ in range(reps):
+        lib.probe_mfma(4096, 4000, sink)
+    _sync()
+    n, k = 2 * cfg["intermediate_size"], cfg["hidden_size"]
+    w = torch.empty(n, k, device=dev, dtype=bf).normal_(0, 0.02)
+    x = torch.randn(tokens, k, device=dev, dtype=bf)
+    out = torch.empty(tokens, n // 2, device=dev, dtype=bf)
+    for _ in range(reps):
+        lib.gemm_bf16(x, w, out, 1, w_frag=False)
+    _sync()
+    wf = torch.empty_like(w)
+    lib.place_rows(w, wf, frag=True)
+    x8, o8 = x[:8].contiguous(), torch.empty(8, n // 2, device=dev, dtype=bf)
+    for _ in range(reps):
+        lib.gemm_bf16_few(x8, wf, o8, 1, w_frag=True)
+    _sync()
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="bench")
     ap.add_argument("--gpus", type=int, default=1)
@@ -245,6 +273,9 @@ def main(argv=None) -> int:
     ap.add_argument("--short-prompts", default="", metavar="N,N,...",
                     help="no benchmark line: one prompt of each of these lengths, launched from Python and issued "
                          "from C++ as a recorded step")
+    ap.add_argument("--load-probe", action="store_true",
+                    help="no benchmark line: a few launches in a row of the MFMA probe and of the named shape's gated "
+                         "product with --prefill-tokens and with 8 tokens, for a profiler that counts cycles")
     ap.add_argument("--tokens", default="1,8,64,512,2048", help="token counts of --planner-sweep")
     ap.add_argument("--sweep-detail", default=None, help="--planner-sweep: a file for every candidate's time")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
@@ -268,6 +299,9 @@ def main(argv=None) -> int:
         return 0
     if len(names) != 1:
         ap.error("one --model at a time")
+    if args.load_probe:
+        load_probe(MODELS[names[0]][1], args.prefill_tokens)
+        return 0
 
     import torch
     from .engine import Engine
