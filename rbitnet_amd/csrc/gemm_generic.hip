@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
 typedef __attribute__((ext_vector_type(4))) float gf_f32x4_t;
 
 template <int MB, int R, bool WF>
-__global__ __launch_bounds__(512) void gemm_f32_few_kernel(const float* __restrict__ x, const float* __restrict__ w,
+__global__ __launch_bounds__(256) void gemm_f32_few_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                           float* __restrict__ c, int m, int n, int k) {
   extern __shared__ float red[];      // [waves - 1][R * MB * 4][64]
   constexpr int ACC = R * MB * 4;
@@ -244,17 +244,32 @@ __global__ __launch_bounds__(512) void gemm_f32_few_kernel(const float* __restri
 }
 
 static int g_f32_few = 1;
-extern "C" void rb_tune_f32_few(int on) { g_f32_few = on; }      // experiments only: 0 = the float32 product of few tokens (W as rows) on the vector units
+// experiments only: 0 = the float32 product of few tokens (W as rows) on the vector units; 3 = one row tile a wave whatever the sizes
+extern "C" void rb_tune_f32_few(int on) { g_f32_few = on; }
 
 // One row tile per wave and at most 4 waves: measured at 1 to 16 tokens on the products of the 8B shape with W
 // fragment-major, two row tiles a wave lose everywhere but in the output matrix at 16 tokens (28,672 rows at
 // K = 4096, 8 tokens: 78 us against 93; 4,096 rows at K = 14336: 38 against 54), and 4 waves are as fast as 8
-// or faster (4,096 rows at K = 4096: 13.2 us against 14.4).
+// or faster (4,096 rows at K = 4096: 13.2 us against 14.4).  The kernel is never launched with more.
 template <int MB>
 static void launch_f32_few(const float* x, const float* w, bool w_frag, float* c, int m, int n, int k, hipStream_t s) {
   int n_waves = k / 256;
   if (n_waves < 1) n_waves = 1;
   if (n_waves > 4) n_waves = 4;
+  // From 33 tokens on a wave reads three to four times as many bytes of tokens as of W for every stage: two row
+  // tiles a wave halve that (28,672 rows at K = 4096 with 64 tokens: 220 us against 305; 128,256 rows: 868
+  // against 1,335; with 33 tokens 227 against 262).
+  if constexpr (MB >= 3) {
+    // (such a wave holds 246 registers, so a compute unit runs one workgroup of them: only where that still
+    // gives every compute unit two workgroups and more)
+    if (g_f32_few != 3 && (n + 31) / 32 >= 2 * rb_compute_units()) {
+      const size_t lds2 = (size_t)(n_waves - 1) * 2 * MB * 4 * 64 * sizeof(float);
+      const int grid2 = (n + 31) / 32;
+      if (w_frag) gemm_f32_few_kernel<MB, 2, true><<<grid2, 64 * n_waves, lds2, s>>>(x, w, c, m, n, k);
+      else gemm_f32_few_kernel<MB, 2, false><<<grid2, 64 * n_waves, lds2, s>>>(x, w, c, m, n, k);
+      return;
+    }
+  }
   const size_t lds = (size_t)(n_waves - 1) * MB * 4 * 64 * sizeof(float);
   const int grid = (n + 15) / 16;
   if (w_frag) gemm_f32_few_kernel<MB, 1, true><<<grid, 64 * n_waves, lds, s>>>(x, w, c, m, n, k);

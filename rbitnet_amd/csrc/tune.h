@@ -12,7 +12,7 @@ void rb_tune_compute_units(int n);                              // every planner
 void rb_tune(int rows_per_wave, int waves);                     // skinny product
 void rb_tune_resident(int tiles);                               // skinny product with resident tokens: row tiles per workgroup
 void rb_tune_use_resident(int on);                              // 0: never the resident variant, 2: also below 8192 rows
-void rb_tune_f32_few(int on);                                   // float32 product of few tokens: 0 = on the vector units, not the float32 MFMA
+void rb_tune_f32_few(int on);                                   // float32 product of few tokens: 0 = on the vector units, not the float32 MFMA; 3 = one row tile a wave always
 void rb_tune_use_stream(int on);                                // 0: the skinny product up to 64 tokens
 void rb_tune_tiles(int cfg, int parts);                         // tiled product: tile configuration and K slices
 int rb_tune_plan(int m, int n, int k, int epilogue);            // tiled product: the built-in choice, 100 * cfg + parts

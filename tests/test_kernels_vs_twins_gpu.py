@@ -130,11 +130,12 @@ def test_gemm_generic(lib, twin, m, n, k):
 
 
 @pytest.mark.parametrize("m", [1, 7, 16, 17, 33, 64])
-@pytest.mark.parametrize("n,k", [(1000, 128), (4096, 512), (8208, 256), (160, 4096 + 128), (28672, 384)])
+@pytest.mark.parametrize("n,k", [(1000, 128), (4096, 512), (8208, 256), (160, 4096 + 128), (28672, 384), (16400, 256)])
 def test_gemm_float32_of_few_tokens(lib, twin, m, n, k):
     """The float32 product for up to 64 tokens on the float32 MFMA (K a multiple of 128): row counts
-    that fill no tile of 16, every number of token blocks, one and two row tiles a workgroup, K in 1 to
-    8 waves with uneven shares, and the same product on the vector units."""
+    that fill no tile of 16, every number of token blocks, one and two row tiles a wave (two from 33 tokens
+    and 16,384 rows on; 16,400 rows leave the last workgroup one), K in 1 to 4 waves with uneven shares, and
+    the same product on the vector units."""
     g = _gen(m * 13 + n + k)
     a, w = torch.randn(m, k, generator=g), torch.randn(n, k, generator=g)
     res = _both(lib, twin, "gemm_generic", [a, w, torch.full((m, n), float("nan"))], [2])
