@@ -250,6 +250,68 @@ def load_probe(cfg, tokens: int, reps: int = 12) -> None:
     _sync()
 
 
+def stream_probe(cfg, tokens: int = 8, copies: int = 8) -> dict:
+    """The products of a decode step beside a kernel that only reads as many bytes (csrc/probe.hip, every
+    workgroup walking pieces of its own with non-temporal loads, the best of four grid sizes): what a layer's
+    products could reach at most if the arithmetic, the tokens and the epilogues cost nothing.  Both as a
+    captured graph of `copies` launches over as many different matrices, so that W comes from memory."""
+    import torch
+    from .csrc.lib import kernels
+    lib = kernels()
+    dev, bf = "cuda:0", torch.bfloat16
+
+    def per_launch(fn) -> float:
+        for i in range(copies):
+            fn(i)
+        _sync()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(copies):
+                fn(i)
+        graph.replay()
+        _sync()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(20):
+            graph.replay()
+        end.record()
+        _sync()
+        return start.elapsed_time(end) / 20 / copies * 1e3
+
+    e, f, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    d = cfg.get("head_dim") or e // cfg["num_attention_heads"]
+    qd, kd = cfg["num_attention_heads"] * d, cfg["num_key_value_heads"] * d
+    sink = torch.zeros(1, device=dev)
+    out = {}
+    for name, n, k, kind in (("qkv", qd + 2 * kd, e, "prepared"), ("o_proj", e, qd, "to_stream"),
+                             ("gate_up", 2 * f, e, "gated"), ("down", e, f, "to_stream"), ("output", v, e, "prepared")):
+        ws = []
+        for _ in range(copies):
+            w = torch.empty(n, k, device=dev, dtype=bf).normal_(0, 0.02)
+            wf = torch.empty_like(w)
+            lib.place_rows(w, wf, frag=True)
+            ws.append(wf)
+            del w
+        a = torch.randn(tokens, k, device=dev).to(bf)
+        squares = torch.rand(tokens, (k + 15) // 16, device=dev) * 16
+        if kind == "to_stream":
+            c, gain = torch.zeros(tokens, n, device=dev), torch.ones(n, device=dev)
+            gained, sq = torch.empty(tokens, n, dtype=bf, device=dev), torch.empty(tokens, (n + 15) // 16, device=dev)
+            fn = lambda i: lib.gemm_bf16_few(a, ws[i], c, 3, gain=gain, gained=gained, squares_out=sq, w_frag=True)
+        elif kind == "gated":
+            c = torch.empty(tokens, n // 2, dtype=bf, device=dev)
+            fn = lambda i: lib.gemm_bf16_few(a, ws[i], c, 1, squares=squares, eps=1e-5, w_frag=True)
+        else:
+            c = torch.empty(tokens, n, device=dev)
+            fn = lambda i: lib.gemm_bf16_few(a, ws[i], c, 0, squares=squares, eps=1e-5, w_frag=True)
+        product = per_launch(fn)
+        views = [w.view(torch.int32) for w in ws]
+        read = min(per_launch(lambda i: lib.probe_read(views[i], sink, blocks, True)) for blocks in (512, 1024, 2048, 4096))
+        out[name] = {"mb": round(n * k * 2 / 1e6, 1), "product_us": round(product, 2), "read_us": round(read, 2)}
+        del ws, views
+    return out
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="bench")
     ap.add_argument("--gpus", type=int, default=1)
@@ -276,6 +338,9 @@ def main(argv=None) -> int:
     ap.add_argument("--load-probe", action="store_true",
                     help="no benchmark line: a few launches in a row of the MFMA probe and of the named shape's gated "
                          "product with --prefill-tokens and with 8 tokens, for a profiler that counts cycles")
+    ap.add_argument("--stream-probe", action="store_true",
+                    help="no benchmark line: the named shape's decode products of 8 tokens beside a kernel that only "
+                         "reads as many bytes")
     ap.add_argument("--tokens", default="1,8,64,512,2048", help="token counts of --planner-sweep")
     ap.add_argument("--sweep-detail", default=None, help="--planner-sweep: a file for every candidate's time")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
@@ -301,6 +366,9 @@ def main(argv=None) -> int:
         ap.error("one --model at a time")
     if args.load_probe:
         load_probe(MODELS[names[0]][1], args.prefill_tokens)
+        return 0
+    if args.stream_probe:
+        print(json.dumps(stream_probe(MODELS[names[0]][1])))
         return 0
 
     import torch
