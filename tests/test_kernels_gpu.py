@@ -712,6 +712,33 @@ def test_products_of_the_model_shapes_with_the_planner_s_own_choice(lib, m, n, k
     assert torch.equal(rows, terms)
 
 
+@pytest.mark.parametrize("units", [40, 96, 304])
+def test_products_planned_for_another_number_of_compute_units(lib, units):
+    """The planners told that the GPU has 40, 96 or 304 compute units (the count is their only input of the
+    machine): other tiles, K slices, rows per wave and workgroup counts, the same products."""
+    from helpers import fragment_major
+    lib._lib.rb_tune_compute_units(units)
+    try:
+        for m, n, k, gated in ((1, 6144, 4096, False), (8, 28672, 4096, True), (16, 4096, 14336, False),
+                               (40, 4096, 4096, False), (64, 512, 14336, False), (200, 12288, 1024, False),
+                               (700, 22016, 2048, True), (1100, 4096, 8192, False)):
+            g = torch.Generator().manual_seed(units + m + n + k)
+            a = torch.randn(m, k, generator=g).bfloat16().to(DEV)
+            w = (torch.randn(n, k, generator=g) * 0.05).bfloat16().to(DEV)
+            wf = fragment_major(w)
+            if gated:
+                out = torch.full((m, n // 2), float("nan"), device=DEV, dtype=torch.bfloat16)
+                lib.gemm_bf16(a, wf, out, 1, w_frag=True)
+                wr = w.float().view(n // 32, 2, 16, k)
+                want = torch.nn.functional.silu(a.float() @ wr[:, 0].reshape(n // 2, k).T) * (a.float() @ wr[:, 1].reshape(n // 2, k).T)
+                assert _rel(out, want) < 1e-2, (units, m, n, k)
+            else:
+                terms = lib.gemm_bf16_terms(a, wf, w_frag=True)
+                assert _rel(terms.sum(0), a.float() @ w.float().T) < 2e-3, (units, m, n, k, terms.shape[0])
+    finally:
+        lib._lib.rb_tune_compute_units(0)
+
+
 @pytest.mark.parametrize("cfg", [4, 5, 6, 7, 8, 9, 10, 13])
 def test_every_tile_of_the_direct_to_lds_product_at_sizes_that_fill_none(lib, cfg):
     """The planner picks a tile by the product's sizes, so sizes of a test reach only some of the
