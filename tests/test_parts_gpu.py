@@ -77,6 +77,49 @@ def test_feed_forward_part(lib, dtype, tol):
         assert got.dtype == torch.float32 and _rel(got, want) < tol, (hidden, ff)
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 8e-3)])
+@pytest.mark.parametrize("style", ["interleaved", "half"])
+def test_position_part(lib, dtype, tol, style):
+    """The rotation part alone: two sequences on unequal pasts bring unequal pieces; q comes back rotated, the
+    rotated k and the plain v lie in the cache at the tokens' positions, with the llama3 rule's three ranges of
+    frequencies in play (positions beyond the original 32)."""
+    hq, hk, d = 3, 2, 24
+    scaling = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+               "original_max_position_embeddings": 32}
+    part = build_part("position", PartSpec("rope", {"head_dim": d, "theta": 500000.0, "scaling": scaling, "style": style,
+                                                    "max_positions": 512}), _env(lib, 48, dtype))
+    cache = Cache([CacheRequest("kv", heads=hk, head_dim=d, window=None)], 2, 64 * 8, dtype, DEV)
+    slots = [cache.alloc_slot(), cache.alloc_slot()]
+    cache.reserve(slots, [70, 3])
+    cache.commit(slots, [70, 3])                       # what lies there already is not read here
+    q_lens = [5, 66]
+    ctx = _step(cache, slots, q_lens)
+    view = cache.view(0, ctx.block_tables)
+    n = sum(q_lens)
+    qkv = torch.randn(n, (hq + 2 * hk) * d)
+    q = torch.empty(n, hq, d, dtype=dtype, device=DEV)
+    part.encode_and_store(qkv.to(DEV), q, view.k_pages, view.v_pages, ctx, view.block_table, hq, hk, d)
+    inv = P.rope_inv_freq(d, 500000.0, scaling)
+    positions = [70 + i for i in range(5)] + [3 + i for i in range(66)]
+    seq_of = [0] * 5 + [1] * 66
+    tables = cache.block_tables(slots)
+    pages = tables[next(iter(tables))]
+    kp, vp = view.k_pages.cpu().double(), view.v_pages.cpu().double()
+    worst = 0.0
+    for t, (pos, b) in enumerate(zip(positions, seq_of)):
+        row = qkv[t].double()
+        for h in range(hq):
+            want = P.rope(row[h * d:(h + 1) * d], pos, inv, style)
+            worst = max(worst, float((q[t, h].double().cpu() - want).abs().max() / want.abs().max()))
+        page, at = pages[b][pos // 64], pos % 64
+        for h in range(hk):
+            want_k = P.rope(row[(hq + h) * d:(hq + h + 1) * d], pos, inv, style)
+            want_v = row[(hq + hk + h) * d:(hq + hk + h + 1) * d]
+            worst = max(worst, float((kp[page, h, at] - want_k).abs().max() / want_k.abs().max()))
+            worst = max(worst, float((vp[page, h, at] - want_v).abs().max() / want_v.abs().max().clamp_min(1e-30)))
+    assert worst < tol
+
+
 def _attention_params(hq, hk, d, window=None, theta=10000.0, style="interleaved", scaling=None):
     return {"num_heads": hq, "num_kv_heads": hk, "head_dim": d, "scale": 1 / math.sqrt(d), "window": window,
             "cache_from": None,
