@@ -120,6 +120,42 @@ def test_position_part(lib, dtype, tol, style):
     assert worst < tol
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 8e-3)])
+@pytest.mark.parametrize("tied", [False, True])
+def test_the_two_ends_alone(lib, dtype, tol, tied):
+    """The embedding part (rows of the table by token id) and the head part (the final norm and the output
+    matrix on the asked rows only, with a pending term still to be added; tied: the embedding's table)."""
+    hidden, vocab = 40, 333
+    env = _env(lib, hidden, dtype)
+    emb = build_part("embedding", PartSpec("table", {"name": "emb.weight", "vocab_size": vocab}), env)
+    head = build_part("head", PartSpec("linear", {"norm": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-4}),
+                                                  "norm_name": "final.weight", "name": None if tied else "out.weight",
+                                                  "vocab_size": vocab}), env)
+    assert set(emb.tensor_specs()) == {"emb.weight"}
+    assert set(head.tensor_specs()) == ({"final.weight"} if tied else {"final.weight", "out.weight"})
+    table = (torch.randn(vocab, hidden) * 0.5).to(dtype)
+    out_w = (torch.randn(vocab, hidden) * 0.5).to(dtype)
+    gain = 1 + 0.2 * torch.randn(hidden)
+    emb.load({"emb.weight": table.to(DEV)})
+    head.load({"final.weight": gain.to(DEV), "out.weight": out_w.to(DEV)}, embedding=emb)
+    ids = [5, 332, 0, 17, 17, 200, 9]
+    ctx = StepContext.for_batch(DEV, StepBatch([0, 1], [0, 0], [ids[:4], ids[4:]], [3, 6], {}),
+                                n_compute_units=lib.n_compute_units)
+    x = emb.forward(ctx)
+    assert x.dtype == torch.float32 and torch.equal(x.cpu(), table[ids].float())
+    pending = (torch.randn(len(ids), hidden) * 0.3).to(DEV)
+    want_rows = (x.cpu().double() + pending.cpu().double())[[3, 6]]
+    logits = head.forward(x, pending, ctx.rows, ctx)
+    w = (table if tied else out_w).double()
+    want = P.linear(P.rmsnorm(want_rows, gain.double(), 1e-4), w)
+    assert logits.dtype == torch.float32 and logits.shape == (2, vocab)
+    assert _rel(logits, want) < tol
+    from rbitnet_amd.errors import ConfigError
+    if tied:
+        with pytest.raises(ConfigError, match="share"):
+            head.load({"final.weight": gain.to(DEV)}, embedding=None)
+
+
 def _attention_params(hq, hk, d, window=None, theta=10000.0, style="interleaved", scaling=None):
     return {"num_heads": hq, "num_kv_heads": hk, "head_dim": d, "scale": 1 / math.sqrt(d), "window": window,
             "cache_from": None,
