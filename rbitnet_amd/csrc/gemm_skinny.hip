@@ -363,7 +363,9 @@ static int launch_skinny(const GemmTokens& x, const bf16_t* w, void* c, const Ge
 // How K is dealt to the waves of a workgroup.  Fast path: K = 128 * T, the T stages dealt to
 // the waves as evenly as they go.  Otherwise the checked path with up to 8 waves.  Measured on the Llama-3-8B
 // products at M = 1..8: one stage in flight per wave (U = 1) is as fast as 2 or 4, and 4
-// waves beat 8 at K = 4096, 8 beat 4 at K = 14336.
+// waves beat 8 at K = 4096, 8 beat 4 at K = 14336.  (With W fragment-major again: launched alone, products
+// with K = 8192 and more gain up to 10 % from two or four stages in flight; the decode steps they belong to
+// lose 4-6 % at the 8B and 70B shapes and gain 1-2 % at hidden sizes of 2,048 and 3,072.  One stage it stays.)
 template <int MB, int R, int EPI, typename TO, bool SCALED>
 static int launch_skinny_u(const GemmTokens& x, const bf16_t* w, void* c, const GemmAfter& after, int m, int n, int k,
                            hipStream_t s) {
